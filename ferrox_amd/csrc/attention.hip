@@ -43,6 +43,8 @@ struct AttnArgs {
     const float* sinks;  // [n_heads] or null: a logit per head that joins the softmax's denominator
     const void* gate;    // [tokens, n_heads * vd] or null (type of out): the output is multiplied by sigmoid(gate)
     long ldg;
+    float softcap;       // > 0: a scaled score s becomes softcap * tanh(s / softcap)
+    const float* slopes; // [n_heads] or null: the score of key t for the query at p then loses slopes[h] * (p - t)
     int bs_shift;        // log2(bs) if bs is a power of two, else -1
     int n_items;
     float scale;
@@ -64,6 +66,12 @@ __device__ __forceinline__ int first_visible(const AttnArgs& a, int p) {
     if (a.mask_chunk > 0) return p - p % a.mask_chunk;
     return a.window > 0 ? max(0, p - a.window + 1) : 0;
 }
+// A scaled score on its way into the softmax: capped, then less the head's penalty for the distance p - t.
+__device__ __forceinline__ float shaped_score(const AttnArgs& a, float slope, float s, int distance) {
+    if (a.softcap > 0.f) s = a.softcap * tanhf(s / a.softcap);
+    return fmaf(-slope, (float)distance, s);
+}
+__host__ __device__ __forceinline__ bool shapes_scores(const AttnArgs& a) { return a.softcap > 0.f || a.slopes != nullptr; }
 // whether queries see a bounded stretch of keys (a window or a chunk) rather than all before them
 __device__ __forceinline__ bool bounded_keys(const AttnArgs& a) { return a.window > 0 || a.mask_chunk > 0; }
 
@@ -188,6 +196,8 @@ __global__ __launch_bounds__(64) void attn_tile_kernel(AttnArgs a) {
     const int kv_end = pmax + 1;
     const KeySpan span = {kv_begin, kv_end, a.keep_first};
     const TileWalk walk = tile_walk(span);
+    const bool shaped = shapes_scores(a);
+    const float slope = a.slopes ? a.slopes[h] : 0.f;
 
     float m[TQ], l[TQ], o[HD_MAX / 64][TQ];
 #pragma unroll
@@ -218,6 +228,7 @@ __global__ __launch_bounds__(64) void attn_tile_kernel(AttnArgs a) {
 #pragma unroll
         for (int i = 0; i < TQ; ++i) {
             const bool vis = in_range && t <= pos[i] && (t >= first_visible(a, pos[i]) || t < a.keep_first);
+            if (shaped) s[i] = shaped_score(a, slope, s[i], pos[i] - t);
             const float sv = vis ? s[i] : NEG_INF;
             const float m_new = fmaxf(m[i], wave_max(sv));
             al[i] = (m_new == NEG_INF) ? 1.f : expf(m[i] - m_new);
@@ -298,6 +309,7 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(AttnArgs a) {
             const T* kr = key_row<T>(a, bt, kvh, t);
             for (int d = 0; d < hd; ++d) s = fmaf(Qs[d], to_float(kr[d]), s);
         }
+        if (shapes_scores(a)) s = shaped_score(a, a.slopes ? a.slopes[h] : 0.f, s, p - t);
         const float sv = vis ? s : NEG_INF;
         const float m_new = fmaxf(m, wave_max(sv));
         const float al = (m_new == NEG_INF) ? 1.f : expf(m - m_new);
@@ -1230,8 +1242,10 @@ FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void*
                          const void* k_pages, const void* v_pages, const int* block_table, int max_blocks,
                          const int* positions, const int* item_seq, const int* item_tok, const int* item_n,
                          int n_items, int nh, int nkv, int hd, int bs, int window, float scale, int tile_q,
-                         int vd, int mask_chunk, int keep_first, const float* sinks, const void* gate, long ldg) {
+                         int vd, int mask_chunk, int keep_first, const float* sinks, const void* gate, long ldg,
+                         float softcap, const float* slopes) {
     if (vd <= 0) vd = hd;
+    FX_REQUIRE(softcap >= 0.f && softcap < INFINITY, "attn_tiles: a cap of %g on the scores", (double)softcap);
     if (check_common("attn_tiles", dtype, nh, nkv, hd, bs, window, scale, vd, mask_chunk, keep_first)) return 1;
     FX_REQUIRE(tile_q == 64 || (tile_q == 128 && wide_items_ok(dtype, hd, bs) && mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages, vd)),
                "attn_tiles: items of %d queries (64, or 128 where fx_attn_tile_queries says so)", tile_q);
@@ -1243,6 +1257,7 @@ FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void*
     a.nh = nh; a.nkv = nkv; a.hd = hd; a.bs = bs; a.window = window; a.scale = scale;
     a.vd = vd; a.mask_chunk = mask_chunk;
     a.keep_first = window > 0 ? keep_first : 0; a.sinks = sinks; a.gate = gate; a.ldg = ldg;
+    a.softcap = softcap; a.slopes = slopes;
     a.bs_shift = log2_or_minus_one(bs);
     a.n_items = n_items;
     dim3 grid(n_items * 4, nh), grid_blocks(8 * ceil_div((long)n_items * nh, 8));     // a wave per 16 queries / a block per item
@@ -1253,7 +1268,7 @@ FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void*
     const bool two_groups = g_groups ? g_groups == 2 : (long)n_items * nh <= fx_compute_units();
     if (dtype == FX_F32)
         attn_tile_kernel<float><<<grid, 64, 0, s>>>(a);
-    else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages, vd)) {
+    else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages, vd) && !shapes_scores(a)) {
         if (tile_q == 128 && hd == 128 && two_groups) attn_mfma_direct_kernel<128, 2, 8, 2><<<grid_blocks, 1024, 0, s>>>(a);
         else if (tile_q == 128 && hd == 64 && two_groups) attn_mfma_direct_kernel<64, 2, 8, 2><<<grid_blocks, 1024, 0, s>>>(a);
         else if (tile_q == 128 && hd == 128) attn_mfma_direct_kernel<128, 2, 8><<<grid_blocks, 512, 0, s>>>(a);
@@ -1280,9 +1295,11 @@ static int attn_decode_launch(void* stream, int dtype, const void* q, long ldq, 
                               const int* positions, const int* item_seq, const int* item_tok, int n_items,
                               int nh, int nkv, int hd, int bs, int window, float scale,
                               float* part_o, float* part_ml, int splits, int chunk, int waves, int vd = 0, int mask_chunk = 0,
-                              int keep_first = 0, const float* sinks = nullptr, const void* gate = nullptr, long ldg = 0) {
+                              int keep_first = 0, const float* sinks = nullptr, const void* gate = nullptr, long ldg = 0,
+                              float softcap = 0.f, const float* slopes = nullptr) {
     if (vd <= 0) vd = hd;
     AttnArgs a = {};
+    a.softcap = softcap; a.slopes = slopes;
     a.q = q; a.ldq = ldq; a.out = out; a.ldo = ldo; a.k_pages = k_pages; a.v_pages = v_pages;
     a.block_table = block_table; a.max_blocks = max_blocks; a.positions = positions;
     a.item_seq = item_seq; a.item_tok = item_tok; a.item_n = nullptr;
@@ -1296,7 +1313,7 @@ static int attn_decode_launch(void* stream, int dtype, const void* q, long ldq, 
     if (dtype == FX_F32) {
         attn_decode_kernel<float><<<grid, 64, 0, s>>>(a);
         attn_decode_merge_kernel<float><<<grid2, 128, splits * sizeof(float), s>>>(a);
-    } else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages, vd)) {
+    } else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages, vd) && !shapes_scores(a)) {
         const int group = nh / nkv;
         dim3 gridm(nkv * ((group + 15) / 16), n_items, splits);
         // as many waves per block (up to 8, and no more than a split has tiles) as their results fit in LDS
@@ -1343,13 +1360,14 @@ FX_API int fx_attn_decode(void* stream, int dtype, const void* q, long ldq, void
                           const int* positions, const int* item_seq, const int* item_tok, int n_items,
                           int nh, int nkv, int hd, int bs, int window, float scale,
                           float* part_o, float* part_ml, int splits, int chunk, int waves, int vd, int mask_chunk,
-                          int keep_first, const float* sinks, const void* gate, long ldg) {
+                          int keep_first, const float* sinks, const void* gate, long ldg, float softcap, const float* slopes) {
     if (attn_decode_check(dtype, nh, nkv, hd, bs, window, scale, splits, chunk)) return 1;
+    FX_REQUIRE(softcap >= 0.f && softcap < INFINITY, "attn_decode: a cap of %g on the scores", (double)softcap);
     if (check_common("attn_decode", dtype, nh, nkv, hd, bs, window, scale, vd, mask_chunk, keep_first)) return 1;
     if (n_items <= 0) return 0;
     return attn_decode_launch(stream, dtype, q, ldq, out, ldo, k_pages, v_pages, block_table, max_blocks, positions,
                               item_seq, item_tok, n_items, nh, nkv, hd, bs, window, scale, part_o, part_ml, splits,
-                              chunk, waves, vd, mask_chunk, keep_first, sinks, gate, ldg);
+                              chunk, waves, vd, mask_chunk, keep_first, sinks, gate, ldg, softcap, slopes);
 }
 
 // ---------------------------------------------------------------------------

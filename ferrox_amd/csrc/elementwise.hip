@@ -9,11 +9,12 @@
 FX_DEFINE_LAST_ERROR()
 
 // ---------------------------------------------------------------------------
-// embedding: h[t, :] = table[ids[t], :]   (no scale; ferrox-models/src/decoder.rs:1279-1284)
+// embedding: h[t, :] = table[ids[t], :] * scale   (the reference has no scale, ferrox-models/src/decoder.rs:1279-1284;
+// a design that multiplies its embeddings by a constant does so here, in float32)
 // ---------------------------------------------------------------------------
 template <typename W>
 __global__ void embed_kernel(const W* __restrict__ table, const int* __restrict__ ids,
-                             float* __restrict__ h, int H, int V) {
+                             float* __restrict__ h, int H, int V, float scale) {
     const int t = blockIdx.x;
     int id = ids[t];
     if (id < 0 || id >= V) {  // the host rejects such ids; never read outside the table
@@ -21,18 +22,18 @@ __global__ void embed_kernel(const W* __restrict__ table, const int* __restrict_
         return;
     }
     const W* row = table + (size_t)id * H;
-    for (int c = threadIdx.x; c < H; c += blockDim.x) h[(size_t)t * H + c] = to_float(row[c]);
+    for (int c = threadIdx.x; c < H; c += blockDim.x) h[(size_t)t * H + c] = to_float(row[c]) * scale;
 }
 
 FX_API int fx_embed(void* stream, int w_dtype, const void* table, const int* ids, float* h,
-                    int T, int H, int V) {
+                    int T, int H, int V, float scale) {
     FX_REQUIRE(T >= 0 && H > 0 && V > 0, "embed: bad sizes T=%d H=%d V=%d", T, H, V);
     if (T == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     if (w_dtype == FX_F32)
-        embed_kernel<float><<<T, 256, 0, s>>>((const float*)table, ids, h, H, V);
+        embed_kernel<float><<<T, 256, 0, s>>>((const float*)table, ids, h, H, V, scale);
     else if (w_dtype == FX_BF16)
-        embed_kernel<bf16><<<T, 256, 0, s>>>((const bf16*)table, ids, h, H, V);
+        embed_kernel<bf16><<<T, 256, 0, s>>>((const bf16*)table, ids, h, H, V, scale);
     else
         return fx_fail("embed: unknown table dtype %d", w_dtype);
     FX_CHECK_LAUNCH("embed");
@@ -48,10 +49,10 @@ FX_API int fx_embed(void* stream, int w_dtype, const void* table, const int* ids
 template <typename T>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ h, const int* __restrict__ rows,
                                                       const void* __restrict__ w, int w_dtype,
-                                                      T* __restrict__ out, int H, float eps) {
+                                                      T* __restrict__ out, int H, float eps, long ld) {
     __shared__ float red[4];
     const int r = blockIdx.x;
-    const float* x = h + (size_t)(rows ? rows[r] : r) * H;
+    const float* x = h + (size_t)(rows ? rows[r] : r) * ld;
     if (H <= 256 * 16) {   // the row stays in registers: one pass over memory, the weights fetched meanwhile
         float xv[16], wv[16];
         float ss = 0.f;
@@ -92,10 +93,10 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
 template <typename T>
 __global__ __launch_bounds__(256) void rmsnorm_short_kernel(const float* __restrict__ h, const int* __restrict__ rows,
                                                             const void* __restrict__ w, int w_dtype,
-                                                            T* __restrict__ out, int R, int H, float eps) {
+                                                            T* __restrict__ out, int R, int H, float eps, long ld) {
     const int r = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
     if (r >= R) return;
-    const float* x = h + (size_t)(rows ? rows[r] : r) * H;
+    const float* x = h + (size_t)(rows ? rows[r] : r) * ld;
     float xv[4], wv[4];
     float ss = 0.f;
 #pragma unroll
@@ -119,22 +120,25 @@ __global__ __launch_bounds__(256) void rmsnorm_short_kernel(const float* __restr
     }
 }
 
+// `ld`: distance between two input rows in floats (0: H, rows that follow each other); the output rows are dense.
 FX_API int fx_rmsnorm(void* stream, int out_dtype, const float* h, const int* rows, const void* w,
-                      int w_dtype, void* out, int R, int H, float eps) {
+                      int w_dtype, void* out, int R, int H, float eps, long ld) {
     FX_REQUIRE(R >= 0 && H > 0, "rmsnorm: bad sizes R=%d H=%d", R, H);
+    if (ld == 0) ld = H;
+    FX_REQUIRE(ld >= H, "rmsnorm: rows %ld apart hold fewer than %d columns", ld, H);
     FX_REQUIRE(w_dtype == FX_F32 || w_dtype == FX_BF16, "rmsnorm: unknown weight dtype %d", w_dtype);
     if (R == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     if (H <= 256 && (out_dtype == FX_F32 || out_dtype == FX_BF16)) {
-        if (out_dtype == FX_F32) rmsnorm_short_kernel<float><<<(R + 3) / 4, 256, 0, s>>>(h, rows, w, w_dtype, (float*)out, R, H, eps);
-        else rmsnorm_short_kernel<bf16><<<(R + 3) / 4, 256, 0, s>>>(h, rows, w, w_dtype, (bf16*)out, R, H, eps);
+        if (out_dtype == FX_F32) rmsnorm_short_kernel<float><<<(R + 3) / 4, 256, 0, s>>>(h, rows, w, w_dtype, (float*)out, R, H, eps, ld);
+        else rmsnorm_short_kernel<bf16><<<(R + 3) / 4, 256, 0, s>>>(h, rows, w, w_dtype, (bf16*)out, R, H, eps, ld);
         FX_CHECK_LAUNCH("rmsnorm");
         return 0;
     }
     if (out_dtype == FX_F32)
-        rmsnorm_kernel<float><<<R, 256, 0, s>>>(h, rows, w, w_dtype, (float*)out, H, eps);
+        rmsnorm_kernel<float><<<R, 256, 0, s>>>(h, rows, w, w_dtype, (float*)out, H, eps, ld);
     else if (out_dtype == FX_BF16)
-        rmsnorm_kernel<bf16><<<R, 256, 0, s>>>(h, rows, w, w_dtype, (bf16*)out, H, eps);
+        rmsnorm_kernel<bf16><<<R, 256, 0, s>>>(h, rows, w, w_dtype, (bf16*)out, H, eps, ld);
     else
         return fx_fail("rmsnorm: unknown output dtype %d", out_dtype);
     FX_CHECK_LAUNCH("rmsnorm");
@@ -387,6 +391,188 @@ FX_API int fx_head_norm_kv_write(void* stream, int dtype, const float* qk, long 
     else
         return fx_fail("head_norm_kv_write: unknown dtype %d", dtype);
     FX_CHECK_LAUNCH("head_norm_kv_write");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Latent attention, what a layer keeps per position.  `down` [T, R + rd] float32 is the down-projection of a
+// token: R latent channels, then a key part of rd dimensions that all heads share.  One block per token:
+//   c = down[:R] / sqrt(mean(down[:R]^2) + eps) * w          (statistics and product in float32)
+//   kr = the key part with the pairs (2i, 2i+1), i < rot / 2, turned by pos * inv_freq[i] and stretched by
+//        `magnitude` (cosine and sine are both multiplied by it); dimensions from rot on pass
+// The key page [page][1][slot][R + rd] receives (c | kr): a query row (its part that went through the keys'
+// up-projection | its rotated part) then scores against it as against the key of one shared head.  The value
+// page [page][1][R][slot] receives c transposed: the heads' outputs are sums of latents, which the values'
+// up-projection is applied to afterwards.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void latent_kv_write_kernel(
+    const float* __restrict__ down, long ldd, const void* __restrict__ w, int w_dtype, float eps,
+    const int* __restrict__ positions, const int* __restrict__ token_seq, const int* __restrict__ block_table, int max_blocks,
+    T* __restrict__ k_pages, T* __restrict__ v_pages, int R, int rd, int rot, int bs, const float* __restrict__ inv_freq,
+    float magnitude) {
+    __shared__ float red[4];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const float* x = down + (size_t)t * ldd;
+    const int pos = positions[t];
+    const int page = block_table[(size_t)token_seq[t] * max_blocks + pos / bs], slot = pos % bs;
+    T* k_dst = k_pages + ((size_t)page * bs + slot) * (R + rd);
+    T* v_dst = v_pages + (size_t)page * R * bs + slot;        // + channel * bs
+    float ss = 0.f;
+    for (int c = tid; c < R; c += 256) ss = fmaf(x[c], x[c], ss);
+    ss = block_sum<4>(ss, red);
+    const float scale = 1.0f / sqrtf(ss / (float)R + eps);
+    for (int c = tid; c < R; c += 256) {
+        T y;
+        from_float(&y, x[c] * scale * load_as_float(w, w_dtype, c));
+        k_dst[c] = y;
+        v_dst[(size_t)c * bs] = y;
+    }
+    const int half = rot >> 1;
+    for (int p = tid; p < half; p += 256) {
+        float sn, cs, y0, y1;
+        sincosf((float)pos * inv_freq[p], &sn, &cs);
+        rotate_pair(x[R + 2 * p], x[R + 2 * p + 1], cs * magnitude, sn * magnitude, y0, y1);
+        from_float(k_dst + R + 2 * p, y0);
+        from_float(k_dst + R + 2 * p + 1, y1);
+    }
+    for (int d = rot + tid; d < rd; d += 256) from_float(k_dst + R + d, x[R + d]);
+}
+
+FX_API int fx_latent_kv_write(void* stream, int dtype, const float* down, long ldd, const void* w, int w_dtype, float eps,
+                              const int* positions, const int* token_seq, const int* block_table, int max_blocks,
+                              void* k_pages, void* v_pages, int T, int R, int rd, int rot, int bs, const float* inv_freq,
+                              float magnitude) {
+    FX_REQUIRE(T >= 0 && R > 0 && rd >= 0 && bs > 0 && ldd >= R + rd, "latent_kv_write: bad sizes T=%d R=%d rd=%d", T, R, rd);
+    FX_REQUIRE(rot >= 0 && rot <= rd && rot % 2 == 0, "latent_kv_write: %d rotated dimensions of %d", rot, rd);
+    FX_REQUIRE(inv_freq || rot == 0, "latent_kv_write: a rotation needs the table of its %d frequencies", rot / 2);
+    FX_REQUIRE(w_dtype == FX_F32 || w_dtype == FX_BF16, "latent_kv_write: unknown weight dtype %d", w_dtype);
+    FX_REQUIRE(k_pages && v_pages && w, "latent_kv_write: pages and the norm's weight are needed");
+    if (T == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == FX_F32)
+        latent_kv_write_kernel<float><<<T, 256, 0, s>>>(down, ldd, w, w_dtype, eps, positions, token_seq, block_table, max_blocks,
+                                                        (float*)k_pages, (float*)v_pages, R, rd, rot, bs, inv_freq, magnitude);
+    else if (dtype == FX_BF16)
+        latent_kv_write_kernel<bf16><<<T, 256, 0, s>>>(down, ldd, w, w_dtype, eps, positions, token_seq, block_table, max_blocks,
+                                                       (bf16*)k_pages, (bf16*)v_pages, R, rd, rot, bs, inv_freq, magnitude);
+    else
+        return fx_fail("latent_kv_write: unknown dtype %d", dtype);
+    FX_CHECK_LAUNCH("latent_kv_write");
+    return 0;
+}
+
+// The rotated part of the queries of latent attention: q [T, nh * (D + rd)] holds per head D dimensions that are
+// not rotated and rd that are; the rd are turned as the shared key part is (pairs (2i, 2i+1), i < rot / 2, by
+// pos * inv_freq[i], stretched by `magnitude`) and written behind the first R columns of that head's row of
+// q_lat [T, nh * (R + rd)] (the first R columns receive the unrotated part times the keys' up-projection from a
+// matrix product).  One block per token.
+template <typename T>
+__global__ __launch_bounds__(256) void latent_q_rot_kernel(const T* __restrict__ q, long ldq, T* __restrict__ q_lat, long ldl,
+                                                           const int* __restrict__ positions, int nh, int D, int rd, int rot, int R,
+                                                           const float* __restrict__ inv_freq, float magnitude) {
+    __shared__ float cs[128], sn[128];
+    const int t = blockIdx.x, tid = threadIdx.x, half = rot >> 1;
+    const int pos = positions[t];
+    for (int p = tid; p < half; p += 256) {
+        float s_, c_;
+        sincosf((float)pos * inv_freq[p], &s_, &c_);
+        cs[p] = c_ * magnitude;
+        sn[p] = s_ * magnitude;
+    }
+    __syncthreads();
+    for (int i = tid; i < nh * half; i += 256) {
+        const int h = i / half, p = i - h * half;
+        const T* src = q + (size_t)t * ldq + (size_t)h * (D + rd) + D;
+        T* dst = q_lat + (size_t)t * ldl + (size_t)h * (R + rd) + R;
+        float y0, y1;
+        rotate_pair(to_float(src[2 * p]), to_float(src[2 * p + 1]), cs[p], sn[p], y0, y1);
+        from_float(dst + 2 * p, y0);
+        from_float(dst + 2 * p + 1, y1);
+    }
+    const int rest = rd - rot;
+    for (int i = tid; i < nh * rest; i += 256) {
+        const int h = i / rest, d = rot + i - h * rest;
+        q_lat[(size_t)t * ldl + (size_t)h * (R + rd) + R + d] = q[(size_t)t * ldq + (size_t)h * (D + rd) + D + d];
+    }
+}
+
+FX_API int fx_latent_q_rot(void* stream, int dtype, const void* q, long ldq, void* q_lat, long ldl, const int* positions,
+                           int T, int nh, int D, int rd, int rot, int R, const float* inv_freq, float magnitude) {
+    FX_REQUIRE(T >= 0 && nh > 0 && D >= 0 && rd >= 0 && R > 0, "latent_q_rot: bad sizes");
+    FX_REQUIRE(ldq >= (long)nh * (D + rd) && ldl >= (long)nh * (R + rd), "latent_q_rot: rows shorter than %d heads", nh);
+    FX_REQUIRE(rot >= 0 && rot <= rd && rot % 2 == 0 && rot <= 256, "latent_q_rot: %d rotated dimensions of %d", rot, rd);
+    FX_REQUIRE(inv_freq || rot == 0, "latent_q_rot: a rotation needs the table of its %d frequencies", rot / 2);
+    if (T == 0 || rd == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == FX_F32)
+        latent_q_rot_kernel<float><<<T, 256, 0, s>>>((const float*)q, ldq, (float*)q_lat, ldl, positions, nh, D, rd, rot, R, inv_freq, magnitude);
+    else if (dtype == FX_BF16)
+        latent_q_rot_kernel<bf16><<<T, 256, 0, s>>>((const bf16*)q, ldq, (bf16*)q_lat, ldl, positions, nh, D, rd, rot, R, inv_freq, magnitude);
+    else
+        return fx_fail("latent_q_rot: unknown dtype %d", dtype);
+    FX_CHECK_LAUNCH("latent_q_rot");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Queries and keys normed over their whole projection, keys that are their own values.  From the float32 product
+// qk [T, nh * hd + nkv * hd] (a token's queries, then its keys), one launch writes
+//   q_out [T, nh * hd]: the queries normed over all nh * hd columns, x / sqrt(mean + eps) * wq[column]
+//   the key page: the keys normed over all nkv * hd columns with wk
+//   the transposed value page: the keys as they are, not normed
+// Blocks (token, 0) take the queries, blocks (token, 1) the keys (left out when there are no pages to write).
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void span_norm_kv_write_kernel(
+    const float* __restrict__ qk, long ldqk, T* __restrict__ q_out, long ldq, const void* __restrict__ wq,
+    const void* __restrict__ wk, int w_dtype, float eps,
+    const int* __restrict__ positions, const int* __restrict__ token_seq, const int* __restrict__ block_table, int max_blocks,
+    T* __restrict__ k_pages, T* __restrict__ v_pages, int nh, int nkv, int hd, int bs) {
+    __shared__ float red[4];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const bool keys = blockIdx.y == 1;
+    const int n = (keys ? nkv : nh) * hd;
+    const float* x = qk + (size_t)t * ldqk + (keys ? (size_t)nh * hd : 0);
+    const void* w = keys ? wk : wq;
+    float ss = 0.f;
+    for (int c = tid; c < n; c += 256) ss = fmaf(x[c], x[c], ss);
+    ss = block_sum<4>(ss, red);
+    const float scale = 1.0f / sqrtf(ss / (float)n + eps);
+    if (!keys) {
+        for (int c = tid; c < n; c += 256) from_float(q_out + (size_t)t * ldq + c, x[c] * scale * load_as_float(w, w_dtype, c));
+        return;
+    }
+    const int pos = positions[t];
+    const int page = block_table[(size_t)token_seq[t] * max_blocks + pos / bs], slot = pos % bs;
+    for (int c = tid; c < n; c += 256) {
+        const int g = c / hd, d = c - g * hd;
+        from_float(k_pages + (((size_t)page * nkv + g) * bs + slot) * hd + d, x[c] * scale * load_as_float(w, w_dtype, c));
+        from_float(v_pages + (((size_t)page * nkv + g) * hd + d) * bs + slot, x[c]);
+    }
+}
+
+FX_API int fx_span_norm_kv_write(void* stream, int dtype, const float* qk, long ldqk, void* q_out, long ldq, const void* wq,
+                                 const void* wk, int w_dtype, float eps, const int* positions, const int* token_seq,
+                                 const int* block_table, int max_blocks, void* k_pages, void* v_pages, int T, int nh, int nkv,
+                                 int hd, int bs) {
+    FX_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && hd > 0 && bs > 0, "span_norm_kv_write: bad sizes");
+    FX_REQUIRE(ldq >= (long)nh * hd && ldqk >= (long)(nh + (k_pages ? nkv : 0)) * hd, "span_norm_kv_write: rows shorter than their heads");
+    FX_REQUIRE(w_dtype == FX_F32 || w_dtype == FX_BF16, "span_norm_kv_write: unknown weight dtype %d", w_dtype);
+    FX_REQUIRE((k_pages == nullptr) == (v_pages == nullptr), "span_norm_kv_write: key and value pages must come together");
+    FX_REQUIRE(wq && (wk || !k_pages), "span_norm_kv_write: the norms' weights are needed");
+    if (T == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid(T, k_pages ? 2 : 1);
+    if (dtype == FX_F32)
+        span_norm_kv_write_kernel<float><<<grid, 256, 0, s>>>(qk, ldqk, (float*)q_out, ldq, wq, wk, w_dtype, eps, positions, token_seq,
+                                                              block_table, max_blocks, (float*)k_pages, (float*)v_pages, nh, nkv, hd, bs);
+    else if (dtype == FX_BF16)
+        span_norm_kv_write_kernel<bf16><<<grid, 256, 0, s>>>(qk, ldqk, (bf16*)q_out, ldq, wq, wk, w_dtype, eps, positions, token_seq,
+                                                             block_table, max_blocks, (bf16*)k_pages, (bf16*)v_pages, nh, nkv, hd, bs);
+    else
+        return fx_fail("span_norm_kv_write: unknown dtype %d", dtype);
+    FX_CHECK_LAUNCH("span_norm_kv_write");
     return 0;
 }
 

@@ -113,6 +113,8 @@ FX_API int fx_short_conv(void* stream, const float* x, long ldx, float* y, long 
 // projections of the gates (all float32):
 //   qn = q / sqrt(sum(q^2) + 1e-6) * D^-1/2,  kn = k / sqrt(sum(k^2) + 1e-6)        per q/k head
 //   decay[h, i] = exp(-exp(A_log[h]) * softplus(a[h, i] + dt_bias[h, i]))             per head and key channel
+//                 (per_head: a and dt_bias hold one number a head, a[h] and dt_bias[h], and all D channels of a
+//                 head receive the same decay)
 //   beta[h] = sigmoid(b[h])
 //   kq[g] = kn[g] . qn[g]                                                             per q/k head (the recurrence needs it per token)
 // Blocks (token, part): part p makes 256 of the token's decays and, a wave each, heads 4p .. 4p+3 of q and k (a
@@ -124,7 +126,8 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(const float* __restr
                                                             const float* __restrict__ a, long lda, const float* __restrict__ b, long ldb,
                                                             const void* __restrict__ A_log, const void* __restrict__ dt_bias, int w_dtype,
                                                             float* __restrict__ qn, float* __restrict__ kn, float* __restrict__ decay,
-                                                            float* __restrict__ beta, float* __restrict__ kq, int H, int G, int D) {
+                                                            float* __restrict__ beta, float* __restrict__ kq, int H, int G, int D,
+                                                            int per_head) {
     const int t = blockIdx.x, part = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     for (int g = part * 4 + wave; g < G; g += 4 * gridDim.y) {          // a wave per head of q and k
         const float* qs = q + (size_t)t * ldq + (size_t)g * D;
@@ -147,9 +150,9 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(const float* __restr
         if (lane == 0) kq[(size_t)t * G + g] = dot;
     }
     for (int idx = part * 256 + threadIdx.x; idx < H * D; idx += 256 * gridDim.y) {
-        const int h = idx / D;
+        const int h = idx / D, src = per_head ? h : idx;
         const float rate = expf(load_as_float(A_log, w_dtype, h));
-        const float step = softplus_f(a[(size_t)t * lda + idx] + load_as_float(dt_bias, w_dtype, idx));
+        const float step = softplus_f(a[(size_t)t * lda + src] + load_as_float(dt_bias, w_dtype, src));
         decay[(size_t)t * H * D + idx] = expf(-rate * step);
     }
     if (part == 0)
@@ -158,13 +161,13 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(const float* __restr
 
 FX_API int fx_delta_prepare(void* stream, const float* q, long ldq, const float* k, long ldk, const float* a, long lda,
                             const float* b, long ldb, const void* A_log, const void* dt_bias, int w_dtype, float* qn,
-                            float* kn, float* decay, float* beta, float* kq, int T, int H, int G, int D) {
+                            float* kn, float* decay, float* beta, float* kq, int T, int H, int G, int D, int per_head) {
     FX_REQUIRE(T >= 0 && H > 0 && G > 0 && D > 0 && H % G == 0, "delta_prepare: bad sizes T=%d H=%d G=%d D=%d", T, H, G, D);
     FX_REQUIRE(w_dtype == FX_F32 || w_dtype == FX_BF16, "delta_prepare: unknown dtype %d", w_dtype);
     if (T == 0) return 0;
     const int parts = (int)fminl(1024, fmaxl((H * (long)D + 255) / 256, (G + 3) / 4));
     delta_prepare_kernel<<<dim3(T, parts), 256, 0, (hipStream_t)stream>>>(q, ldq, k, ldk, a, lda, b, ldb, A_log, dt_bias, w_dtype, qn, kn,
-                                                             decay, beta, kq, H, G, D);
+                                                             decay, beta, kq, H, G, D, per_head);
     FX_CHECK_LAUNCH("delta_prepare");
     return 0;
 }
@@ -407,12 +410,13 @@ FX_API int fx_channel_delta(void* stream, const float* qn, const float* kn, cons
 
 // ---------------------------------------------------------------------------
 // The read-out's way to the output projection: every head's o is divided by its root mean square over V
-// (eps inside the root), times a weight shared by the heads, times sigmoid(gate[h, :]).  One wave per (token, head).
+// (eps inside the root), times a weight shared by the heads, times sigmoid(gate[h, :]) (gate_act 0) or
+// silu(gate[h, :]) (gate_act 1).  One wave per (token, head).
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void gated_head_norm_kernel(const float* __restrict__ o, long ldo, const float* __restrict__ gate,
                                                               long ldg, const void* __restrict__ w, int w_dtype, T* __restrict__ y,
-                                                              long ldy, int n_rows, int H, int V, float eps) {
+                                                              long ldy, int n_rows, int H, int V, float eps, int gate_act) {
     const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
     if (row >= n_rows) return;
     const int t = row / H, h = row - t * H;
@@ -422,13 +426,15 @@ __global__ __launch_bounds__(256) void gated_head_norm_kernel(const float* __res
     ss = wave_sum(ss);
     const float scale = 1.0f / sqrtf(ss / (float)V + eps);
     for (int i = lane; i < V; i += 64) {
-        const float gt = 1.0f / (1.0f + expf(-gate[(size_t)t * ldg + (size_t)h * V + i]));
+        const float gx = gate[(size_t)t * ldg + (size_t)h * V + i];
+        const float gt = (gate_act ? gx : 1.0f) / (1.0f + expf(-gx));
         from_float(y + (size_t)t * ldy + (size_t)h * V + i, src[i] * scale * load_as_float(w, w_dtype, i) * gt);
     }
 }
 
 FX_API int fx_gated_head_norm(void* stream, int out_dtype, const float* o, long ldo, const float* gate, long ldg,
-                              const void* w, int w_dtype, void* y, long ldy, int T, int H, int V, float eps) {
+                              const void* w, int w_dtype, void* y, long ldy, int T, int H, int V, float eps, int gate_act) {
+    FX_REQUIRE(gate_act == 0 || gate_act == 1, "gated_head_norm: gate activation %d (0 sigmoid, 1 silu)", gate_act);
     FX_REQUIRE(T >= 0 && H > 0 && V > 0, "gated_head_norm: bad sizes T=%d H=%d V=%d", T, H, V);
     FX_REQUIRE(w_dtype == FX_F32 || w_dtype == FX_BF16, "gated_head_norm: unknown weight dtype %d", w_dtype);
     FX_REQUIRE((long)T * H < (1L << 31), "gated_head_norm: too many rows for one launch");
@@ -436,9 +442,9 @@ FX_API int fx_gated_head_norm(void* stream, int out_dtype, const float* o, long 
     const int rows = T * H;
     hipStream_t s = (hipStream_t)stream;
     if (out_dtype == FX_F32)
-        gated_head_norm_kernel<float><<<(rows + 3) / 4, 256, 0, s>>>(o, ldo, gate, ldg, w, w_dtype, (float*)y, ldy, rows, H, V, eps);
+        gated_head_norm_kernel<float><<<(rows + 3) / 4, 256, 0, s>>>(o, ldo, gate, ldg, w, w_dtype, (float*)y, ldy, rows, H, V, eps, gate_act);
     else if (out_dtype == FX_BF16)
-        gated_head_norm_kernel<bf16><<<(rows + 3) / 4, 256, 0, s>>>(o, ldo, gate, ldg, w, w_dtype, (bf16*)y, ldy, rows, H, V, eps);
+        gated_head_norm_kernel<bf16><<<(rows + 3) / 4, 256, 0, s>>>(o, ldo, gate, ldg, w, w_dtype, (bf16*)y, ldy, rows, H, V, eps, gate_act);
     else
         return fx_fail("gated_head_norm: unknown output dtype %d", out_dtype);
     FX_CHECK_LAUNCH("gated_head_norm");

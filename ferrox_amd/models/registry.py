@@ -86,6 +86,9 @@ def _register_builtin():
     from ..config.kovalorn import KovalornConfig
     from .kovalorn import build_spec as kovalorn_spec
     register_architecture(Architecture(KovalornConfig.architecture, KovalornConfig.model_type, KovalornConfig, kovalorn_spec))
+    from ..config.fokinex import FokinexConfig
+    from .fokinex import build_spec as fokinex_spec
+    register_architecture(Architecture(FokinexConfig.architecture, FokinexConfig.model_type, FokinexConfig, fokinex_spec))
 
 
 _register_builtin()

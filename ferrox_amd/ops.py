@@ -59,8 +59,16 @@ def _stream():
 
 
 _sigs = {
-    ("elementwise", "fx_embed"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int],
-    ("elementwise", "fx_rmsnorm"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float],
+    ("elementwise", "fx_embed"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float],
+    ("elementwise", "fx_latent_kv_write"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_int, c_float, c_void_p, c_void_p,
+                                            c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p,
+                                            c_float],
+    ("elementwise", "fx_latent_q_rot"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_int, c_int,
+                                         c_int, c_int, c_int, c_void_p, c_float],
+    ("elementwise", "fx_span_norm_kv_write"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_int,
+                                               c_float, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int,
+                                               c_int, c_int, c_int],
+    ("elementwise", "fx_rmsnorm"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_long],
     ("elementwise", "fx_rope_kv_write"): [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
                                           c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                                           c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int],
@@ -71,13 +79,13 @@ _sigs = {
                                      c_void_p, c_void_p, c_void_p, c_int, c_int, c_int],
     ("recurrent", "fx_delta_prepare"): [c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_long, c_void_p, c_long,
                                         c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                        c_int, c_int, c_int, c_int],
+                                        c_int, c_int, c_int, c_int, c_int],
     ("recurrent", "fx_channel_delta"): [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long,
                                         c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int],
     ("recurrent", "fx_small_rows_pair"): [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_int,
                                           c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_int, c_int],
     ("recurrent", "fx_gated_head_norm"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_void_p,
-                                          c_long, c_int, c_int, c_int, c_float],
+                                          c_long, c_int, c_int, c_int, c_float, c_int],
     ("elementwise", "fx_head_norm_kv_write"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int,
                                                c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p, c_int,
                                                c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int],
@@ -96,13 +104,13 @@ _sigs = {
     ("attention", "fx_attn_tiles"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p,
                                      c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int,
-                                     c_int, c_void_p, c_void_p, c_long],
+                                     c_int, c_void_p, c_void_p, c_long, c_float, c_void_p],
     ("attention", "fx_attn_tile_queries"): [c_int, c_int, c_int],
     ("attention", "fx_attn_decode"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p,
                                       c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                                       c_int, c_int, c_int, c_int, c_int, c_float,
                                       c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                                      c_int, c_void_p, c_void_p, c_long],
+                                      c_int, c_void_p, c_void_p, c_long, c_float, c_void_p],
     ("moe", "fx_router_select"): [c_void_p, c_void_p, c_long, c_long, c_int, c_int, c_int, c_int, c_float, c_float, c_int,
                                   c_void_p, c_void_p, c_void_p, c_void_p],
     ("moe", "fx_router_select_align"): [c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_float, c_float, c_int,
@@ -141,30 +149,34 @@ def _i32(t, what):
 
 
 # ---------------------------------------------------------------------------
-def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
-    """h[t] = table[ids[t]] as float32."""
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | None = None, scale: float = 1.0) -> torch.Tensor:
+    """h[t] = table[ids[t]] * scale as float32."""
     V, H = table.shape
     T = ids.numel()
     if out is None:
         out = torch.empty((T, H), dtype=torch.float32, device=table.device)
-    _call("elementwise", "fx_embed", _stream(), dtype_code(table.dtype), _p(table), _p(_i32(ids, "ids")), _p(out), T, H, V)
+    _call("elementwise", "fx_embed", _stream(), dtype_code(table.dtype), _p(table), _p(_i32(ids, "ids")), _p(out), T, H, V,
+          float(scale))
     return out
 
 
 def rmsnorm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
-            rows: torch.Tensor | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
+            rows: torch.Tensor | None = None, out: torch.Tensor | None = None, width: int | None = None) -> torch.Tensor:
     """Rows of float32 `h` (all, or those in `rows`) normed into `out_dtype`; `weight` None: brought to unit root
-    mean square, no more."""
-    if h.dtype != torch.float32 or not h.is_contiguous():
-        raise KernelError("rmsnorm reads a contiguous float32 residual stream")
-    H = h.shape[-1]
+    mean square, no more.  `width`: the norm runs over the first so many columns of every row (the rows may then be
+    any distance apart); the output is dense [rows, width]."""
+    if h.dtype != torch.float32 or h.dim() != 2 or h.stride(1) != 1 or (width is None and not h.is_contiguous()):
+        raise KernelError("rmsnorm reads float32 rows with unit inner stride (contiguous ones unless `width` is given)")
+    H = h.shape[-1] if width is None else int(width)
+    if not 0 < H <= h.shape[-1]:
+        raise KernelError(f"rmsnorm: a width of {H} for rows of {h.shape[-1]}")
     if weight is not None and weight.numel() != H:
         raise KernelError(f"rmsnorm weight has {weight.numel()} elements for width {H}")
     R = h.shape[0] if rows is None else rows.numel()
     if out is None:
         out = torch.empty((R, H), dtype=out_dtype, device=h.device)
     _call("elementwise", "fx_rmsnorm", _stream(), dtype_code(out_dtype), _p(h), _p(_i32(rows, "rows")), _p(weight),
-          dtype_code(weight.dtype) if weight is not None else FX_F32, _p(out), R, H, float(eps))
+          dtype_code(weight.dtype) if weight is not None else FX_F32, _p(out), R, H, float(eps), h.stride(0))
     return out
 
 
@@ -265,6 +277,99 @@ def head_norm_kv_write(qk, q_out, v, q_weight, k_weight, eps, positions, token_s
           float(eps), _p(_i32(positions, "positions")), _p(_i32(token_seq, "token_seq")),
           _p(_i32(block_table, "block_table")), block_table.shape[1] if block_table is not None else 0,
           _p(k_pages), _p(v_pages) if with_keys else None, T, n_heads, n_kv_heads, head_dim, block_size, v_dim)
+
+
+
+def latent_kv_write(down, weight, eps, positions, token_seq, block_table, k_pages, v_pages, kv_rank: int, rot_dim: int,
+                    rotary_dim: int, block_size: int, inv_freq, magnitude: float = 1.0) -> None:
+    """What a latent-attention layer keeps per position, from the float32 down-projection `down` [T, kv_rank +
+    rot_dim]: the first kv_rank columns through an RMS norm with `weight` (the latent c), the last rot_dim with the
+    pairs (2i, 2i+1), i < rotary_dim / 2, turned by pos * inv_freq[i] and stretched by `magnitude`.  The key page
+    [pages, 1, block_size, kv_rank + rot_dim] receives (c | rotated part), the value page [pages, 1, kv_rank,
+    block_size] c transposed."""
+    T = down.shape[0]
+    R, rd = int(kv_rank), int(rot_dim)
+    _f32_rows(down, "latent_kv_write: the down-projection", R + rd)
+    if weight.numel() != R or not weight.is_contiguous():
+        raise KernelError(f"latent_kv_write: a norm weight of {weight.numel()} elements for a latent of {R}")
+    if k_pages.dtype != v_pages.dtype or tuple(k_pages.shape[1:]) != (1, block_size, R + rd) or \
+            tuple(v_pages.shape[1:]) != (1, R, block_size) or not k_pages.is_contiguous() or not v_pages.is_contiguous():
+        raise KernelError(f"latent_kv_write: pages {tuple(k_pages.shape)}, {tuple(v_pages.shape)}; expected "
+                          f"[pages,1,{block_size},{R + rd}] and [pages,1,{R},{block_size}]")
+    if rotary_dim and (inv_freq is None or inv_freq.dtype != torch.float32 or inv_freq.numel() != rotary_dim // 2):
+        raise KernelError(f"latent_kv_write: {rotary_dim} rotated dimensions need {rotary_dim // 2} float32 frequencies")
+    if positions.numel() < T or token_seq.numel() < T:
+        raise KernelError("latent_kv_write: the step's index tensors are shorter than its tokens")
+    _call("elementwise", "fx_latent_kv_write", _stream(), dtype_code(k_pages.dtype), _p(down), down.stride(0), _p(weight),
+          dtype_code(weight.dtype), float(eps), _p(_i32(positions, "positions")), _p(_i32(token_seq, "token_seq")),
+          _p(_i32(block_table, "block_table")), block_table.shape[1], _p(k_pages), _p(v_pages), T, R, rd, int(rotary_dim),
+          int(block_size), _p(inv_freq), float(magnitude))
+
+
+def latent_q_rot(q, q_lat, positions, n_heads: int, dim: int, rot_dim: int, rotary_dim: int, kv_rank: int, inv_freq,
+                 magnitude: float = 1.0) -> None:
+    """The rotated part of latent attention's queries: the last rot_dim dimensions of every head of q [T, n_heads *
+    (dim + rot_dim)], turned as `latent_kv_write` turns the shared key part, go behind the first kv_rank columns of
+    that head's row of q_lat [T, n_heads * (kv_rank + rot_dim)]."""
+    T = q.shape[0]
+    for t, cols, what in ((q, n_heads * (dim + rot_dim), "q"), (q_lat, n_heads * (kv_rank + rot_dim), "q_lat")):
+        if t.dim() != 2 or t.stride(1) != 1 or t.shape[1] < cols or t.shape[0] < T or t.dtype != q.dtype:
+            raise KernelError(f"latent_q_rot: {what} {tuple(t.shape)} for {n_heads} heads")
+    if rotary_dim and (inv_freq is None or inv_freq.dtype != torch.float32 or inv_freq.numel() != rotary_dim // 2):
+        raise KernelError(f"latent_q_rot: {rotary_dim} rotated dimensions need {rotary_dim // 2} float32 frequencies")
+    if positions.numel() < T:
+        raise KernelError("latent_q_rot: fewer positions than tokens")
+    _call("elementwise", "fx_latent_q_rot", _stream(), dtype_code(q.dtype), _p(q), q.stride(0), _p(q_lat), q_lat.stride(0),
+          _p(_i32(positions, "positions")), T, int(n_heads), int(dim), int(rot_dim), int(rotary_dim), int(kv_rank),
+          _p(inv_freq), float(magnitude))
+
+
+def span_norm_kv_write(qk, q_out, q_weight, k_weight, eps, positions, token_seq, block_table, k_pages, v_pages,
+                       n_heads: int, n_kv_heads: int, head_dim: int, block_size: int) -> None:
+    """Queries and keys normed over their whole projection, keys that are their own values, in one launch: from the
+    float32 product qk [T, (n_heads + n_kv_heads) * head_dim], the queries go, normed over all their columns with
+    `q_weight` (one element a column), to q_out [T, n_heads * head_dim]; the keys, normed over all theirs with
+    `k_weight`, into the key page, and as they are into the transposed value page (`k_pages` None: q alone, and qk
+    may hold the queries only)."""
+    T = qk.shape[0]
+    qw, kw = int(n_heads) * int(head_dim), int(n_kv_heads) * int(head_dim)
+    with_keys = k_pages is not None
+    _f32_rows(qk, "span_norm_kv_write: the q/k product", qw + (kw if with_keys else 0))
+    if q_out.stride(-1) != 1 or q_out.shape[0] < T or q_out.shape[1] < qw:
+        raise KernelError(f"span_norm_kv_write: q_out {tuple(q_out.shape)} for {T} tokens of {qw} columns")
+    if q_weight.numel() != qw or not q_weight.is_contiguous():
+        raise KernelError(f"span_norm_kv_write: a query norm weight of {q_weight.numel()} elements for rows of {qw}")
+    if with_keys:
+        if k_weight is None or k_weight.numel() != kw or not k_weight.is_contiguous() or k_weight.dtype != q_weight.dtype:
+            raise KernelError(f"span_norm_kv_write: the key norm's weight must hold {kw} elements of the query norm's type")
+        if k_pages.dtype != q_out.dtype or v_pages.dtype != q_out.dtype or \
+                tuple(k_pages.shape[1:]) != (n_kv_heads, block_size, head_dim) or \
+                tuple(v_pages.shape[1:]) != (n_kv_heads, head_dim, block_size) or not k_pages.is_contiguous() or not v_pages.is_contiguous():
+            raise KernelError(f"span_norm_kv_write: pages {tuple(k_pages.shape)}, {tuple(v_pages.shape)} ({k_pages.dtype})")
+    if positions.numel() < T or token_seq.numel() < T:
+        raise KernelError("span_norm_kv_write: the step's index tensors are shorter than its tokens")
+    _call("elementwise", "fx_span_norm_kv_write", _stream(), dtype_code(q_out.dtype), _p(qk), qk.stride(0), _p(q_out),
+          q_out.stride(0), _p(q_weight), _p(k_weight) if with_keys else None, dtype_code(q_weight.dtype), float(eps),
+          _p(_i32(positions, "positions")), _p(_i32(token_seq, "token_seq")), _p(_i32(block_table, "block_table")),
+          block_table.shape[1] if block_table is not None else 0, _p(k_pages), _p(v_pages) if with_keys else None, T,
+          int(n_heads), int(n_kv_heads), int(head_dim), int(block_size))
+
+
+_constant_rows: dict = {}
+
+
+def constant_rows(device, value: float, n: int) -> torch.Tensor:
+    """float32 [n] on the device, every element `value`: a row scale for products whose output is weighted by a
+    constant (`gemm(..., row_scale=)`).  Tables are kept for the life of the process (recorded steps hold their
+    addresses) and grow in powers of two."""
+    key = (torch.device(device), float(value))
+    have = _constant_rows.setdefault(key, [])
+    for t in have:
+        if t.numel() >= n:
+            return t[:n]
+    size = 1 << max(10, (int(n) - 1).bit_length())
+    have.append(torch.full((size,), float(value), dtype=torch.float32, device=device))
+    return have[-1][:n]
 
 
 def residual_add(h: torch.Tensor, y: torch.Tensor) -> None:
@@ -522,26 +627,34 @@ def attention_tile_queries(dtype, head_dim: int, block_size: int) -> int:
 
 def attention_tiles(q, out, k_pages, v_pages, block_table, positions, item_seq, item_tok, item_n,
                     n_heads, n_kv_heads, head_dim, block_size, window, scale, tile_q: int = 64, mask_chunk: int = 0,
-                    v_dim: int | None = None, keep_first: int = 0, sinks=None, gate=None) -> None:
+                    v_dim: int | None = None, keep_first: int = 0, sinks=None, gate=None, softcap: float = 0.0,
+                    slopes=None) -> None:
     """Blocks of queries: item i is item_n[i] <= tile_q consecutive tokens of sequence item_seq[i] from token
     item_tok[i] on; tile_q is 64 or attention_tile_queries(...).  `mask_chunk` > 0: the chunked mask (a query sees
     the keys of its own chunk of that many positions) instead of a window.  `v_dim`: size of a value head where it
     is not head_dim; `out` is [T, n_heads * v_dim].  `keep_first` (with a window): the first so many keys of a
     sequence stay visible to every later query.  `sinks` (float32 [n_heads]): a logit per head that joins the
-    softmax's denominator and has no value.  `gate` (shape and type of `out`): the output is multiplied by sigmoid(gate)."""
+    softmax's denominator and has no value.  `gate` (shape and type of `out`): the output is multiplied by sigmoid(gate).
+    `softcap` > 0: a scaled score s becomes softcap * tanh(s / softcap).  `slopes` (float32 [n_heads]): the score of
+    key t for the query at position p then loses slopes[h] * (p - t)."""
     _check_attention_shapes(q, out, k_pages, v_pages, n_heads, n_kv_heads, head_dim, int(v_dim or head_dim), block_size)
-    _check_attention_extras(out, n_heads, int(v_dim or head_dim), window, keep_first, sinks, gate)
+    _check_attention_extras(out, n_heads, int(v_dim or head_dim), window, keep_first, sinks, gate, softcap, slopes)
     _call("attention", "fx_attn_tiles", _stream(), dtype_code(q.dtype), _p(q), q.stride(0), _p(out), out.stride(0),
           _p(k_pages), _p(v_pages), _p(_i32(block_table, "block_table")), block_table.shape[1],
           _p(_i32(positions, "positions")), _p(_i32(item_seq, "item_seq")), _p(_i32(item_tok, "item_tok")),
           _p(_i32(item_n, "item_n")), item_seq.numel(), n_heads, n_kv_heads, head_dim, block_size,
           int(window or 0), float(scale), int(tile_q), int(v_dim or head_dim), int(mask_chunk or 0),
-          int(keep_first or 0), _p(sinks), _p(gate), gate.stride(0) if gate is not None else 0)
+          int(keep_first or 0), _p(sinks), _p(gate), gate.stride(0) if gate is not None else 0, float(softcap or 0.0),
+          _p(slopes))
 
 
-def _check_attention_extras(out, n_heads, v_dim, window, keep_first, sinks, gate) -> None:
+def _check_attention_extras(out, n_heads, v_dim, window, keep_first, sinks, gate, softcap=0.0, slopes=None) -> None:
     if keep_first and not window:
         raise KernelError("attention: kept first keys go with a window")
+    if not 0.0 <= float(softcap or 0.0) < math.inf:
+        raise KernelError(f"attention: a cap of {softcap} on the scores")
+    if slopes is not None and (slopes.dtype != torch.float32 or not slopes.is_contiguous() or slopes.numel() != n_heads):
+        raise KernelError(f"attention: distance slopes must be {n_heads} contiguous float32 values")
     if sinks is not None and (sinks.dtype != torch.float32 or not sinks.is_contiguous() or sinks.numel() != n_heads):
         raise KernelError(f"attention: sinks must be {n_heads} contiguous float32 values")
     if gate is not None and (gate.dtype != out.dtype or gate.stride(-1) != 1 or gate.shape[0] < out.shape[0]
@@ -589,7 +702,7 @@ def decode_attention_chunk(n_items: int, n_heads: int, n_kv_heads: int, max_kv_l
 def attention_decode(q, out, k_pages, v_pages, block_table, positions, item_seq, item_tok,
                      n_heads, n_kv_heads, head_dim, block_size, window, scale, max_kv_len, chunk=None,
                      waves=0, mask_chunk: int = 0, v_dim: int | None = None, keep_first: int = 0, sinks=None,
-                     gate=None) -> None:
+                     gate=None, softcap: float = 0.0, slopes=None) -> None:
     """Single queries.  The keys go to ceil(max_kv_len / chunk) blocks whose results are merged in ascending
     order.  float32 cuts them at multiples of `chunk`, 256 by default (so that a result does not depend on the
     batch); bfloat16, whose blocks of up to eight waves share a chunk, cuts every sequence's own range of keys (from
@@ -598,7 +711,7 @@ def attention_decode(q, out, k_pages, v_pages, block_table, positions, item_seq,
     n = item_seq.numel()
     v_dim = int(v_dim or head_dim)
     _check_attention_shapes(q, out, k_pages, v_pages, n_heads, n_kv_heads, head_dim, v_dim, block_size)
-    _check_attention_extras(out, n_heads, v_dim, window, keep_first, sinks, gate)
+    _check_attention_extras(out, n_heads, v_dim, window, keep_first, sinks, gate, softcap, slopes)
     if chunk is None:
         chunk = 256
         if q.dtype == torch.bfloat16:
@@ -611,7 +724,8 @@ def attention_decode(q, out, k_pages, v_pages, block_table, positions, item_seq,
           _p(_i32(positions, "positions")), _p(_i32(item_seq, "item_seq")), _p(_i32(item_tok, "item_tok")), n,
           n_heads, n_kv_heads, head_dim, block_size, int(window or 0), float(scale),
           _p(part_o), _p(part_ml), splits, chunk, int(waves), v_dim, int(mask_chunk or 0),
-          int(keep_first or 0), _p(sinks), _p(gate), gate.stride(0) if gate is not None else 0)
+          int(keep_first or 0), _p(sinks), _p(gate), gate.stride(0) if gate is not None else 0, float(softcap or 0.0),
+          _p(slopes))
 
 
 def router_select(logits, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gate=False, selection_bias=None,
@@ -815,15 +929,17 @@ def short_conv(x, taps, state, token_seq, seq_starts, slot_ids, n_seqs: int) -> 
     return y
 
 
-def delta_prepare(q, k, a, b, A_log, dt_bias, n_heads: int, n_kv_heads: int, key_dim: int):
+def delta_prepare(q, k, a, b, A_log, dt_bias, n_heads: int, n_kv_heads: int, key_dim: int, per_head: bool = False):
     """From convolved q, k [T, G*D], the decay's projection a [T, H*D] and the step size's b [T, H] (float32 rows):
     (q / |q| / sqrt(D), k / |k|, exp(-exp(A_log[h]) softplus(a + dt_bias)), sigmoid(b), the normed k . q per q/k head
-    [T, G]), all float32 contiguous."""
+    [T, G]), all float32 contiguous.  `per_head`: a is [T, H] and dt_bias [H], one decay per head, which all D
+    channels of the head receive (the decays returned are [T, H*D] either way)."""
     T = q.shape[0]
     H, G, D = int(n_heads), int(n_kv_heads), int(key_dim)
+    Dd = 1 if per_head else D
     _f32_rows(q, "delta_prepare: q", G * D), _f32_rows(k, "delta_prepare: k", G * D)
-    _f32_rows(a, "delta_prepare: a", H * D), _f32_rows(b, "delta_prepare: b", H)
-    if A_log.numel() != H or dt_bias.numel() != H * D or A_log.dtype != dt_bias.dtype or not A_log.is_contiguous() \
+    _f32_rows(a, "delta_prepare: a", H * Dd), _f32_rows(b, "delta_prepare: b", H)
+    if A_log.numel() != H or dt_bias.numel() != H * Dd or A_log.dtype != dt_bias.dtype or not A_log.is_contiguous() \
             or not dt_bias.is_contiguous():
         raise KernelError(f"delta_prepare: A_log {tuple(A_log.shape)} / dt_bias {tuple(dt_bias.shape)} for {H} heads of {D}")
     dev = q.device
@@ -833,7 +949,8 @@ def delta_prepare(q, k, a, b, A_log, dt_bias, n_heads: int, n_kv_heads: int, key
     beta = torch.empty((T, H), dtype=torch.float32, device=dev)
     kq = torch.empty((T, G), dtype=torch.float32, device=dev)
     _call("recurrent", "fx_delta_prepare", _stream(), _p(q), q.stride(0), _p(k), k.stride(0), _p(a), a.stride(0), _p(b),
-          b.stride(0), _p(A_log), _p(dt_bias), dtype_code(A_log.dtype), _p(qn), _p(kn), _p(decay), _p(beta), _p(kq), T, H, G, D)
+          b.stride(0), _p(A_log), _p(dt_bias), dtype_code(A_log.dtype), _p(qn), _p(kn), _p(decay), _p(beta), _p(kq), T, H, G, D,
+          1 if per_head else 0)
     return qn, kn, decay, beta, kq
 
 
@@ -858,9 +975,14 @@ def channel_delta(qn, kn, decay, beta, kq, v, state, seq_starts, slot_ids, n_seq
     return out
 
 
-def gated_head_norm(o, gate, weight, eps: float, n_heads: int, v_dim: int, out_dtype) -> torch.Tensor:
-    """y[t, h, :] = o[t, h, :] / rms(o[t, h, :]) * weight * sigmoid(gate[t, h, :]) in `out_dtype`; o and gate are
-    float32 rows [T, H*V], weight [V] is shared by the heads."""
+HEAD_GATES = {"sigmoid": 0, "silu": 1}
+
+
+def gated_head_norm(o, gate, weight, eps: float, n_heads: int, v_dim: int, out_dtype, gate_activation: str = "sigmoid") -> torch.Tensor:
+    """y[t, h, :] = o[t, h, :] / rms(o[t, h, :]) * weight * act(gate[t, h, :]) in `out_dtype`, act being sigmoid or
+    silu; o and gate are float32 rows [T, H*V], weight [V] is shared by the heads."""
+    if gate_activation not in HEAD_GATES:
+        raise KernelError(f"gated_head_norm: gate activation '{gate_activation}' is not one of {sorted(HEAD_GATES)}")
     T = o.shape[0]
     H, V = int(n_heads), int(v_dim)
     _f32_rows(o, "gated_head_norm: o", H * V), _f32_rows(gate, "gated_head_norm: gate", H * V)
@@ -868,7 +990,7 @@ def gated_head_norm(o, gate, weight, eps: float, n_heads: int, v_dim: int, out_d
         raise KernelError(f"gated_head_norm: gate {tuple(gate.shape)} / weight {tuple(weight.shape)} for {T} x {H} heads of {V}")
     y = torch.empty((T, H * V), dtype=out_dtype, device=o.device)
     _call("recurrent", "fx_gated_head_norm", _stream(), dtype_code(out_dtype), _p(o), o.stride(0), _p(gate), gate.stride(0),
-          _p(weight), dtype_code(weight.dtype), _p(y), y.stride(0), T, H, V, float(eps))
+          _p(weight), dtype_code(weight.dtype), _p(y), y.stride(0), T, H, V, float(eps), HEAD_GATES[gate_activation])
     return y
 
 

@@ -70,7 +70,8 @@ class PagedAttention(Mixer):
                  position: PartSpec, window: int | None = None, scale: float | None = None,
                  qk_norm: PartSpec | None = None, v_dim: int | None = None, chunk: int | None = None,
                  names: dict | None = None, keep_first: int = 0, sink: bool = False, out_gate: bool = False,
-                 own_kv: bool = True, retain: tuple | None = None):
+                 own_kv: bool = True, retain: tuple | None = None, softcap: float | None = None,
+                 distance_slopes=None, values_from_keys: bool = False, qk_norm_span: str = "head"):
         """`qk_norm`: kind and arguments of a norm over head_dim; two of them are built, with tensors under
         `q_norm.` and `k_norm.`, and applied to every head of q and of k before the rotation.
         `v_dim`: size of a value head where it differs from head_dim (the size of a query and key head).
@@ -85,7 +86,13 @@ class PagedAttention(Mixer):
         `own_kv` False: the mixer has no key and value projections and writes no cache; its schedule entry reads
         the cache of an entry that has them (with these head counts and sizes).
         `retain` = (window or None, keep_first): how the pages of this mixer's cache group age, where that is not
-        its own mask: the longest window and the most kept keys among the mixers that read the same cache."""
+        its own mask: the longest window and the most kept keys among the mixers that read the same cache.
+        `softcap`: a scaled score s becomes softcap * tanh(s / softcap) before the softmax.
+        `distance_slopes` (n_heads numbers): the score of key t for the query at position p then loses
+        slope_h * (p - t); this is how positions enter the scores of a mixer that rotates nothing.
+        `values_from_keys`: the mixer has no value projection; a key as projected (before any norm) is its value.
+        `qk_norm_span` "projection": the norms of `qk_norm` run over all heads of q at once and over all heads of k at
+        once (weights of n_heads * head_dim and n_kv_heads * head_dim elements) instead of over every head."""
         if n_heads % n_kv_heads:
             raise ValueError(f"n_heads {n_heads} is not a multiple of n_kv_heads {n_kv_heads}")
         # (the matrix-unit kernels take multiples of HEAD_DIM_STEP; other sizes run on the kernels for any shape)
@@ -109,6 +116,22 @@ class PagedAttention(Mixer):
             raise ValueError(f"a cache that keeps the last {self.retain[0]} and the first {self.retain[1]} keys does not hold "
                              f"what a window of {self.window} with {self.keep_first} kept keys sees")
         self.v_dim = int(v_dim) if v_dim else head_dim
+        self.softcap = float(softcap) if softcap else 0.0
+        if not 0.0 <= self.softcap < math.inf:
+            raise ValueError(f"a cap of {softcap} on the scores")
+        self.distance_slopes = tuple(float(x) for x in distance_slopes) if distance_slopes is not None else None
+        if self.distance_slopes is not None and len(self.distance_slopes) != n_heads:
+            raise ValueError(f"{len(self.distance_slopes)} distance slopes for {n_heads} heads")
+        self.values_from_keys = bool(values_from_keys)
+        if self.values_from_keys and (self.v_dim != head_dim or bias):
+            raise ValueError("keys that are their own values have the values' size and no biases")
+        if qk_norm_span not in ("head", "projection"):
+            raise ValueError(f"qk_norm_span '{qk_norm_span}' is not 'head' or 'projection'")
+        self.span_norms = qk_norm_span == "projection"
+        if self.span_norms and qk_norm is None:
+            raise ValueError("norms over the whole projection need `qk_norm`")
+        if self.values_from_keys and not self.span_norms:
+            raise ValueError("keys that are their own values come with norms over the whole projection here")
         if not 1 <= self.v_dim <= limits.HEAD_DIM_MAX:
             raise ValueError(f"v_dim {self.v_dim}: the attention kernels take up to {limits.HEAD_DIM_MAX}")
         self.names = dict(self.TENSORS, **(names or {}))
@@ -122,22 +145,33 @@ class PagedAttention(Mixer):
         self.qw, self.kvw, self.vw, self.ow = n_heads * head_dim, n_kv_heads * head_dim, n_kv_heads * self.v_dim, n_heads * self.v_dim
         if not self.own_kv:
             self.kvw = self.vw = 0       # (no rows of k and v in the mixer's matrix)
-        self.qkv = self.o_proj = self.sinks = None
+        if self.values_from_keys:
+            self.vw = 0                  # (no rows of v: the key rows are the values)
+        self.qkv = self.o_proj = self.sinks = self.slopes = None
         self.q_norm = self.k_norm = None
-        if qk_norm is not None:
+        if qk_norm is not None and self.span_norms:
+            self.q_norm = NORMS.build(PartSpec(qk_norm.kind, dict(qk_norm.args, size=self.qw)))
+            self.k_norm = NORMS.build(PartSpec(qk_norm.kind, dict(qk_norm.args, size=self.kvw))) if self.kvw else None
+            if self.q_norm.rms_params() is None or (self.position.rotary() or Rotary(1, 1.0)).rotary_dim:
+                raise ValueError("norms over the whole projection are RMS norms with a weight, under a mixer that rotates nothing")
+        elif qk_norm is not None:
             self.q_norm, self.k_norm = (NORMS.build(PartSpec(qk_norm.kind, dict(qk_norm.args))) for _ in range(2))
+        if (self.position.rotary() or Rotary(0, 1.0)).magnitude != 1.0:
+            raise ValueError("this mixer's rotation kernels turn and do not stretch: a rotation's magnitude must be 1")
         if bias and out_gate:
             raise ValueError("an attention layer with an output gate has no biases here")
 
     def children(self):
-        norms = [(self.names["q_norm"], self.q_norm), (self.names["k_norm"], self.k_norm)] if self.q_norm is not None else []
+        norms = [(self.names[n], p) for n, p in (("q_norm", self.q_norm), ("k_norm", self.k_norm)) if p is not None]
         return [(self._position_prefix, self.position)] + norms
 
     def param_specs(self):
         H, n = self.hidden_size, self.names
         specs = {n["q"]: ParamSpec((self.qw, H)), n["o"]: ParamSpec((H, self.ow))}
         if self.own_kv:
-            specs.update({n["k"]: ParamSpec((self.kvw, H)), n["v"]: ParamSpec((self.vw, H))})
+            specs[n["k"]] = ParamSpec((self.kvw, H))
+            if not self.values_from_keys:
+                specs[n["v"]] = ParamSpec((self.vw, H))
         if self.bias:
             specs.update({n["q_bias"]: ParamSpec((self.qw,)), n["k_bias"]: ParamSpec((self.kvw,)),
                           n["v_bias"]: ParamSpec((self.vw,))})
@@ -150,7 +184,8 @@ class PagedAttention(Mixer):
     def load(self, fetch):
         # one matrix: the rows of q, then (a mixer with projections of its own) of k and v, then of the output gate
         n = self.names
-        rows = [fetch(n["q"])] + ([fetch(n["k"]), fetch(n["v"])] if self.own_kv else []) \
+        rows = [fetch(n["q"])] + ([fetch(n["k"])] if self.own_kv else []) \
+            + ([fetch(n["v"])] if self.own_kv and not self.values_from_keys else []) \
             + ([fetch(n["gate"])] if self.out_gate else [])
         w = torch.cat(same_dtype(rows), dim=0)
         b = None
@@ -160,7 +195,28 @@ class PagedAttention(Mixer):
         self.o_proj = Linear(fetch(n["o"]))
         if self.has_sink:
             self.sinks = fetch(n["sink"]).float().contiguous()
+        if self.distance_slopes is not None:
+            self.slopes = torch.tensor(self.distance_slopes, dtype=torch.float64).to(torch.float32).to(w.device)
 
+    def normed_spans_and_cache(self, x, ctx, table, cache):
+        """As `normed_heads_and_cache` for norms over the whole projection: q [T, qw] normed over all its columns, the
+        keys normed over all theirs into the key page and, where they are their own values, as projected into the
+        value page, in one launch; returns q and the rest of the product (v, the output gate's rows)."""
+        wq, eps = self.q_norm.rms_params()
+        w = self.qkv.weight
+        cut = self.qw + self.kvw
+        qk = matmul(x, w[:cut], epilogue=ops.EPI_STORE_F32)
+        rest = matmul(x, w[cut:]) if w.shape[0] > cut else None
+        q = torch.empty((ctx.n_tokens, self.qw), dtype=ctx.act_dtype, device=qk.device)
+        writes = self.own_kv and cache.writes
+        if writes and not self.values_from_keys:
+            raise ValueError("norms over the whole projection with a value projection of their own have no kernel yet")
+        debug.region("rope + cache write")
+        wk = self.k_norm.rms_params()[0] if self.k_norm is not None else None
+        ops.span_norm_kv_write(qk, q, wq, wk, eps, ctx.positions, ctx.token_seq, table,
+                               cache.pages["k"] if writes else None, cache.pages["v"] if writes else None,
+                               self.n_heads, self.n_kv_heads, self.head_dim, cache.block_size)
+        return q, rest
 
     def page_shapes(self, block_size: int) -> dict:
         return {"k": (self.n_kv_heads, block_size, self.head_dim),
@@ -271,7 +327,9 @@ class PagedAttention(Mixer):
                                cache.block_size, self.v_dim)
         return q, rest
 
-    def forward(self, x, ctx, cache, residual, qkv=None, post_norm=None) -> None:
+    def forward(self, x, ctx, cache, residual, qkv=None, post_norm=None, out_scale: float | None = None) -> None:
+        """`out_scale`: a constant that the mixer's output is multiplied by on its way into the stream (a mixer that
+        runs beside another one, the two weighted)."""
         table = ctx.block_tables[cache.group]
         k_pages, v_pages = cache.pages["k"], cache.pages["v"]
         rot = self.position.rotary()
@@ -290,7 +348,10 @@ class PagedAttention(Mixer):
             gate = None
             wrote = False
             if self.q_norm is not None:           # every head of q and k through its norm, between bias and rotation
-                if self.fuses_head_norms():
+                if self.span_norms:
+                    q, rest = self.normed_spans_and_cache(x, ctx, table, cache)
+                    k, wrote = None, True
+                elif self.fuses_head_norms():
                     # RMS norms and no rotation: one launch norms the heads and writes q, k's and v's pages
                     q, rest = self.normed_heads_and_cache(x, ctx, table, cache)
                     k, wrote = None, True
@@ -327,7 +388,7 @@ class PagedAttention(Mixer):
         common = (self.n_heads, self.n_kv_heads, self.head_dim, cache.block_size, self.window, self.scale)
         # (the gate multiplies the heads' outputs as the attention kernels write them)
         mask = dict(mask_chunk=self.chunk or 0, v_dim=self.v_dim, keep_first=self.keep_first, sinks=self.sinks,
-                    gate=None if fused else gate)
+                    gate=None if fused else gate, softcap=self.softcap, slopes=self.slopes)
         if items["n_tiles"]:
             ops.attention_tiles(q, out, k_pages, v_pages, table, ctx.positions,
                                 items["tile_seq"], items["tile_tok"], items["tile_n"], *common, tile_q=tile_q, **mask)
@@ -336,6 +397,7 @@ class PagedAttention(Mixer):
                                  items["dec_seq"], items["dec_tok"], *common, max_kv_len=items["max_kv"], **mask)
         debug.region("o_proj")
         if post_norm is None:
-            self.o_proj(out, epilogue=ops.EPI_RESID, out=residual)
+            scale = ops.constant_rows(out.device, out_scale, ctx.n_tokens) if out_scale is not None and out_scale != 1.0 else None
+            self.o_proj(out, epilogue=ops.EPI_RESID, out=residual, row_scale=scale)
         else:       # the output rows are normed before they join the stream: float32 rows, then one kernel norms and adds
             ops.rmsnorm_add(residual, self.o_proj(out, epilogue=ops.EPI_STORE_F32), post_norm[0], post_norm[1])

@@ -236,12 +236,15 @@ class Rotary:
     freq_factors[i] if a table is given (float32 [rotary_dim / 2] on the device).  Pairs are
     (i, i + rotary_dim/2), or (2i, 2i+1) when `interleaved`.  rotary_dim 0 rotates nothing.
     `frequencies` (a tuple of rotary_dim / 2 numbers) replaces theta^(-2i/rotary_dim) by a table of the
-    encoding's own: pair i turns by pos * frequencies[i], the product taken in float32."""
+    encoding's own: pair i turns by pos * frequencies[i], the product taken in float32.
+    `magnitude`: cosine and sine are both multiplied by it (a rotation that also stretches the rotated
+    dimensions); only mixers that say so apply one that is not 1."""
     rotary_dim: int
     theta: float
     interleaved: bool = False
     freq_factors: torch.Tensor | None = None
     frequencies: tuple | None = None
+    magnitude: float = 1.0
 
 
 class PositionEncoding(Part):

@@ -100,3 +100,26 @@ class SandwichBlock(Block):
         if self.ffn is not None:
             debug.region("norm")
             self._sublayer(self.ffn, self.norm2b, self.norm2.forward(h, ctx), ctx, h)
+
+
+@BLOCKS.register("parallel")
+class ParallelBlock(Block):
+    """h += mixer(norm1(h)) + ffn(norm1(h)): one norm, and both sublayers read its output.  A layer without a
+    feed-forward has the mixer only.  Both sublayers end with a product that adds into the float32 stream; the
+    normed rows are made before either has added, so the order of the two additions changes rounding alone."""
+    slots = {"norm1": NORMS, "mixer": MIXERS, "ffn": FEED_FORWARDS}
+    optional_slots = ("ffn",)
+
+    def __init__(self, parts: dict, prefixes: dict):
+        self.norm1, self.mixer, self.ffn = parts["norm1"], parts["mixer"], parts.get("ffn")
+        self._prefixes = prefixes
+
+    def children(self):
+        return [(self._prefixes[s], getattr(self, s)) for s in self.slots if getattr(self, s, None) is not None]
+
+    def forward(self, h, ctx, cache):
+        debug.region("norm")
+        x = self.norm1.forward(h, ctx)
+        self.mixer.forward(x, ctx, cache, h)
+        if self.ffn is not None:
+            self.ffn.forward(x, ctx, h)

@@ -1,7 +1,10 @@
-"""Token embedding (no scale, ferrox-models/src/decoder.rs:1279-1284) and the output
+"""Token embedding (the reference's has no scale, ferrox-models/src/decoder.rs:1279-1284; `scale` multiplies the rows
+of a design that has one) and the output
 head, applied to the wanted rows only (decoder.rs:2994-3009); a tied head shares
 the embedding table (ferrox-models/src/loader.rs:1433-1436)."""
 from __future__ import annotations
+
+import math
 
 from .. import ops
 from .base import EMBEDDINGS, HEADS, ParamSpec, Part
@@ -12,9 +15,13 @@ from .linear import matmul
 class TokenEmbedding(Part):
     kernel_libraries = ("elementwise",)
 
-    def __init__(self, vocab_size: int, hidden_size: int, name: str = "weight"):
+    def __init__(self, vocab_size: int, hidden_size: int, name: str = "weight", scale: float = 1.0):
+        """`scale`: a constant that every embedding row is multiplied by on its way into the float32 stream."""
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.name = name
+        self.scale = float(scale)
+        if not math.isfinite(self.scale):
+            raise ValueError(f"an embedding scale of {scale}")
         self.weight = None
 
     def param_specs(self):
@@ -24,30 +31,31 @@ class TokenEmbedding(Part):
         self.weight = fetch(self.name).contiguous()
 
     def forward(self, token_ids):
-        return ops.embed(self.weight, token_ids)
+        return ops.embed(self.weight, token_ids, scale=self.scale)
 
 
 @HEADS.register("linear_head")
 class LinearHead(Part):
     kernel_libraries = ("gemm",)
 
-    def __init__(self, vocab_size: int, hidden_size: int, tied_to: str | None = None):
-        """`tied_to`: the full name of another part's [vocab, hidden] tensor that serves as this head's matrix (the
+    def __init__(self, vocab_size: int, hidden_size: int, tied_to: str | None = None, name: str = "weight"):
+        """`name`: what the head's own matrix is called behind the part's prefix.  `tied_to`: the full name of another part's [vocab, hidden] tensor that serves as this head's matrix (the
         embedding table of a model with tied embeddings); the head then has no tensor of its own."""
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.tied_to = tied_to or None
+        self.name = name
         self.weight = None
 
     def param_specs(self):
-        return {} if self.tied_to else {"weight": ParamSpec((self.vocab_size, self.hidden_size))}
+        return {} if self.tied_to else {self.name: ParamSpec((self.vocab_size, self.hidden_size))}
 
     def borrows(self):
         return [self.tied_to] if self.tied_to else []
 
     def load(self, fetch):
-        self.weight = (fetch.shared(self.tied_to) if self.tied_to else fetch("weight")).contiguous()
+        self.weight = (fetch.shared(self.tied_to) if self.tied_to else fetch(self.name)).contiguous()
         if tuple(self.weight.shape) != (self.vocab_size, self.hidden_size):
-            raise ValueError(f"the head's matrix {self.tied_to or 'weight'} has shape {tuple(self.weight.shape)}, "
+            raise ValueError(f"the head's matrix {self.tied_to or self.name} has shape {tuple(self.weight.shape)}, "
                              f"not [{self.vocab_size}, {self.hidden_size}]")
 
     def forward(self, x):

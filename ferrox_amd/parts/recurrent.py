@@ -10,6 +10,10 @@ input row:
     y = W_o (o / rms(o) * w_norm * sigmoid(W_g2 (W_g1 h)))                    norm and gate per head
 Value head j reads q/k head j // (heads / kv_heads).  The state S and the convolution's last taps - 1 inputs
 are carried in the request's slot; everything from the convolution to the norm is float32.
+
+`head_delta`: the same rule with one decay per head and full-rank gates:
+    d = exp(-exp(A_log) * softplus(W_a h + dt_bias))                          one decay per head, S <- d S
+    y = W_o (o / rms(o) * w_norm * silu(W_g h))
 """
 from __future__ import annotations
 
@@ -119,5 +123,70 @@ class ChannelDelta(Mixer):
         debug.region("o_proj")
         if post_norm is None:
             self.o_proj(y, epilogue=ops.EPI_RESID, out=residual)
+        else:
+            ops.rmsnorm_add(residual, self.o_proj(y, epilogue=ops.EPI_STORE_F32), post_norm[0], post_norm[1])
+
+
+@MIXERS.register("head_delta")
+class HeadDelta(ChannelDelta):
+    """The gated delta rule with one decay per head (W_a: [heads, hidden], dt_bias: [heads]) and an output gate
+    silu(W_g h) of full rank (W_g: [heads * v_dim, hidden]).  State, convolution, unit vectors, step sizes and the
+    recurrence are `channel_delta`'s, through the same kernels: the decay of a head is handed to all its key channels."""
+    TENSORS = {"q": "q", "k": "k", "v": "v", "q_conv": "q.conv", "k_conv": "k.conv", "v_conv": "v.conv", "beta": "b",
+               "A_log": "A_log", "dt_bias": "dt_bias", "decay": "a", "gate": "g", "norm": "norm", "o": "o"}
+
+    def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, key_dim: int, v_dim: int, conv_taps: int,
+                 norm_eps: float, gate_activation: str = "silu", names: dict | None = None):
+        super().__init__(hidden_size, n_heads, n_kv_heads, key_dim, v_dim, conv_taps, norm_eps, decay_rank=1, gate_rank=1)
+        if gate_activation not in ops.HEAD_GATES:
+            raise ValueError(f"gate activation '{gate_activation}' is not one of {sorted(ops.HEAD_GATES)}")
+        self.gate_activation = gate_activation
+        self.names = dict(self.TENSORS, **(names or {}))
+
+    def param_specs(self):
+        W, n = self.hidden_size, self.names
+        H, t = self.n_heads, self.conv_taps
+        return {
+            n["q"]: ParamSpec((self.qk_width, W)), n["q_conv"]: ParamSpec((self.qk_width, t)),
+            n["k"]: ParamSpec((self.qk_width, W)), n["k_conv"]: ParamSpec((self.qk_width, t)),
+            n["v"]: ParamSpec((self.v_width, W)), n["v_conv"]: ParamSpec((self.v_width, t)),
+            n["beta"]: ParamSpec((H, W)), n["A_log"]: ParamSpec((H,)), n["norm"]: ParamSpec((self.v_dim,), init="ones"),
+            n["decay"]: ParamSpec((H, W)), n["dt_bias"]: ParamSpec((H,)),
+            n["gate"]: ParamSpec((self.v_width, W)), n["o"]: ParamSpec((W, self.v_width)),
+        }
+
+    def load(self, fetch):
+        n = self.names
+        # one product makes everything that reads the input row: q | k | v | beta | decay | gate
+        self.w_in = torch.cat(same_dtype([fetch(n[x]) for x in ("q", "k", "v", "beta", "decay", "gate")]), dim=0).contiguous()
+        self.taps = torch.cat([fetch(n[x]).float() for x in ("q_conv", "k_conv", "v_conv")], dim=0).contiguous()
+        self.A_log = fetch(n["A_log"]).float().contiguous()
+        self.dt_bias = fetch(n["dt_bias"]).float().contiguous()
+        self.norm_w = fetch(n["norm"]).contiguous()
+        self.o_proj = Linear(fetch(n["o"]))
+
+    def forward(self, x, ctx, cache, residual, post_norm=None, out_scale: float | None = None) -> None:
+        H, G, D, V = self.n_heads, self.n_kv_heads, self.key_dim, self.v_dim
+        C, QK = self.conv_channels, self.qk_width
+        debug.region("delta in")
+        proj = matmul(x, self.w_in, epilogue=ops.EPI_STORE_F32)
+        starts = sequence_starts(ctx)
+        o1 = C + H          # beta ends
+        o2 = o1 + H         # decay ends; the gate's rows follow
+        debug.region("delta conv")
+        conv = ops.short_conv(proj[:, :C], self.taps, cache.state["conv"], ctx.token_seq, starts, ctx.slot_ids, ctx.n_seqs)
+        debug.region("delta gates")
+        qn, kn, decay, beta, kq = ops.delta_prepare(conv[:, :QK], conv[:, QK:2 * QK], proj[:, o1:o2], proj[:, C:o1], self.A_log,
+                                                    self.dt_bias, H, G, D, per_head=True)
+        debug.region("delta rule")
+        o = ops.channel_delta(qn, kn, decay, beta, kq, conv[:, 2 * QK:], cache.state["S"], starts, ctx.slot_ids, ctx.n_seqs,
+                              H, G, D, V)
+        debug.region("delta out")
+        y = ops.gated_head_norm(o, proj[:, o2:o2 + self.v_width], self.norm_w, self.norm_eps, H, V, ctx.act_dtype,
+                                gate_activation=self.gate_activation)
+        debug.region("o_proj")
+        if post_norm is None:
+            scale = ops.constant_rows(y.device, out_scale, ctx.n_tokens) if out_scale is not None and out_scale != 1.0 else None
+            self.o_proj(y, epilogue=ops.EPI_RESID, out=residual, row_scale=scale)
         else:
             ops.rmsnorm_add(residual, self.o_proj(y, epilogue=ops.EPI_STORE_F32), post_norm[0], post_norm[1])

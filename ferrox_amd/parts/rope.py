@@ -85,3 +85,51 @@ class ScaledRope(_Rotary):
 
     def rotary(self):
         return Rotary(self.rotary_dim, self.theta, self.interleaved, None, self.frequencies)
+
+
+def ramped_frequencies(rotary_dim: int, theta: float, factor: float, original: float, fast: float, slow: float) -> tuple:
+    """theta^(-2i/rotary_dim) stretched by pair index, in float64.  d(t) = rotary_dim ln(original / (2 pi t)) /
+    (2 ln theta) is the (fractional) pair whose wave makes t turns over `original` positions.  Pairs up to
+    lo = max(floor(d(fast)), 0) keep their frequency f, pairs from hi = min(ceil(d(slow)), rotary_dim - 1) on get
+    f / factor, and between them the two are blended with a ramp (i - lo) / max(hi - lo, 0.001) clamped to [0, 1]."""
+    import math
+
+    def pair_of(turns: float) -> float:
+        return rotary_dim * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(theta))
+
+    lo = max(math.floor(pair_of(fast)), 0)
+    hi = min(math.ceil(pair_of(slow)), rotary_dim - 1)
+    out = []
+    for i in range(rotary_dim // 2):
+        f = float(theta) ** (-2.0 * i / rotary_dim)
+        ramp = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+        out.append(f / factor * ramp + f * (1.0 - ramp))
+    return tuple(out)
+
+
+@POSITION_ENCODINGS.register("rope_ramped")
+class RampedRope(_Rotary):
+    """A rotation for contexts `factor` times longer than the `original` one: frequencies stretched by pair index
+    (`ramped_frequencies`), and cosine and sine both multiplied by 0.1 ln(factor) + 1, which makes up for the
+    scores' loss of contrast under the slower waves.  `scaling` = (factor, original, fast, slow) or None (a plain
+    rotation, magnitude 1).  Either pairing."""
+    MAGNITUDE_SLOPE = 0.1
+
+    def __init__(self, head_dim: int, theta: float, rotary_dim: int | None = None, interleaved: bool = False,
+                 scaling=None):
+        import math
+        super().__init__(head_dim, theta, rotary_dim)
+        self.interleaved = bool(interleaved)
+        self.magnitude = 1.0
+        if scaling is not None:
+            scaling = tuple(float(x) for x in scaling)
+            if len(scaling) != 4 or min(scaling) <= 0 or self.theta == 1.0:
+                raise ValueError(f"ramped rope scaling is (factor, original, fast, slow), all positive, theta not 1; got {scaling}")
+            self.frequencies = ramped_frequencies(self.rotary_dim, self.theta, *scaling) if self.rotary_dim else ()
+            self.magnitude = self.MAGNITUDE_SLOPE * math.log(scaling[0]) + 1.0
+        else:
+            self.frequencies = tuple(self.theta ** (-2.0 * i / self.rotary_dim) for i in range(self.rotary_dim // 2))
+        self.scaling = scaling
+
+    def rotary(self):
+        return Rotary(self.rotary_dim, self.theta, self.interleaved, None, self.frequencies, self.magnitude)
