@@ -439,6 +439,22 @@ __device__ __forceinline__ float quad_sum(float x) {
     return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
+// A lane's 16 raw scores sc[kb][r] of keys key0 + 4*kb + r, scaled, capped and less the head's penalty for the
+// distance from the row's query at qpos (`shaped_score` with a tanh made of one exponential, whose error, some
+// 1e-7 of the cap, is far below what bfloat16 operands leave of a score): afterwards they are scores in natural
+// units, and the softmax step takes them with c = log2(e).
+__device__ __forceinline__ void shape_scores(f32x4_t (&sc)[4], int key0, const AttnArgs& a, float slope, int qpos) {
+    const float inv_cap = a.softcap > 0.f ? 1.f / a.softcap : 0.f;
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float s = sc[kb][r] * a.scale;
+            if (a.softcap > 0.f) s = a.softcap * (1.f - 2.f / (1.f + __expf(2.f * s * inv_cap)));
+            sc[kb][r] = fmaf(-slope, (float)(qpos - (key0 + 4 * kb + r)), s);
+        }
+}
+
 // One step of the one-pass softmax on a lane's 16 raw scores sc[kb][r] of keys key0 + 4*kb + r
 // (key0 = tile start + 16g), in base 2: t = score * c with c = scale * log2(e), m and l are the
 // running maximum (of t) and sum of this lane's row, shared by the row's four lanes.  MASKED: only
@@ -541,12 +557,13 @@ struct WaveAttn {
     }
 
     // keys [kt0, kt0 + 64); this lane's row sees key t iff t <= hi and (lo <= t or t < span.keep) (hi < lo: row unused)
+    // `slope`, `qpos`: the row's distance penalty and its query's position, where the scores are shaped
     __device__ __forceinline__ void tile(const AttnArgs& a, const PageLookup& pl, int kvh, int kt0, const KeySpan& span,
-                                         int lo, int hi) {
+                                         int lo, int hi, float slope = 0.f, int qpos = 0) {
         const int kv_end = span.end;
         const int lane = threadIdx.x & 63, li = lane & 15, g = lane >> 4;
         const int l8 = li & 7, lh = li >> 3;
-        const int hd = a.hd, bs = a.bs;
+        const int hd = a.hd, bs = a.bs, vd = a.vd;      // (vd <= hd: the value heads may be narrower than the key heads)
         // Loads are issued without branches: a key outside [kv_begin, kv_end) (its page may have been
         // given back) reads from a group of keys that is inside, and its data is replaced by zeros.
         const int safe_group = (kv_end - 1) & ~15;
@@ -581,7 +598,7 @@ struct WaveAttn {
             page_slot(a, span.has(key_b) ? key_b : safe_group, kblk, kslots_b[kb]);
             kpage_b[kb] = pl.page(kblk);
         }
-        const bf16* vbase = (const bf16*)a.v_pages + ((size_t)vpage * a.nkv + kvh) * hd * bs + vslot;
+        const bf16* vbase = (const bf16*)a.v_pages + ((size_t)vpage * a.nkv + kvh) * vd * bs + vslot;
         uint4 vv[EARLY_V ? CB : 1][2];
         const uint32_t vmask = opaque_mask(vlive);
         if (EARLY_V) {
@@ -590,8 +607,8 @@ struct WaveAttn {
                 // whole lines: the first load's lanes take rows 16 cb + li % 8, the second's the eight after them, both
                 // the keys 8 (li / 8) .. of the lane's 16; the halves change places before the products
                 const int d1 = 16 * cb + l8, d2 = d1 + 8;
-                vv[cb][0] = load_lines16(vbase + (size_t)(d1 < hd ? d1 : 0) * bs + 8 * lh);
-                vv[cb][1] = load_lines16(vbase + (size_t)(d2 < hd ? d2 : 0) * bs + 8 * lh);
+                vv[cb][0] = load_lines16(vbase + (size_t)(d1 < vd ? d1 : 0) * bs + 8 * lh);
+                vv[cb][1] = load_lines16(vbase + (size_t)(d2 < vd ? d2 : 0) * bs + 8 * lh);
             }
         }
         f32x4_t sc[4];
@@ -602,6 +619,7 @@ struct WaveAttn {
             const bf16* krb = (const bf16*)a.k_pages + (((size_t)kpage_b[kb] * a.nkv + kvh) * bs + kslots_b[kb]) * hd;
 #pragma unroll
             for (int u = 0; u < KP; u += 2) {
+                if (HD > 128 && 32 * u >= hd) continue;           // (the same in every lane: k-steps past the head's size)
                 const int d = 32 * u + 32 * lh + 8 * g;           // the low or the high 32 of the pair's 64
                 kf[kb][u] = load_lines16(kra + (d < hd ? d : 0));
                 kf[kb][u + 1] = load_lines16(krb + (d < hd ? d : 0));
@@ -623,6 +641,7 @@ struct WaveAttn {
             const uint32_t kmask = opaque_mask(klives[kb]);
 #pragma unroll
             for (int u = 0; u < KS; ++u) {
+                if (HD > 128 && 32 * u >= hd) continue;
                 uint4 ku = kf[kb][u];
                 if (u < KP) {
                     // low 32: own first load below lane 8 of a row of 16, the other half's second load above;
@@ -635,7 +654,9 @@ struct WaveAttn {
         }
         // softmax on this lane's 16 scores (keys kt0 + 16g + 4kb + r); the row's four lanes share max and sum
         uint4 p_lo, p_hi;
-        const float alpha = softmax_step<true>(sc, kt0 + 16 * g, lo, hi, a.scale * LOG2E, m, l, p_lo, p_hi, span.keep);
+        const bool shaped = shapes_scores(a);
+        if (shaped) shape_scores(sc, kt0 + 16 * g, a, slope, qpos);
+        const float alpha = softmax_step<true>(sc, kt0 + 16 * g, lo, hi, shaped ? LOG2E : a.scale * LOG2E, m, l, p_lo, p_hi, span.keep);
         const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0;
         float al[4] = {1.f, 1.f, 1.f, 1.f};
         if (rescale) {
@@ -644,6 +665,7 @@ struct WaveAttn {
         }
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) {
+            if (HD > 128 && 16 * cb >= vd) continue;              // (the same in every lane: columns past the value head's size)
             uint4 v0, v1;
             {
                 uint4 t1, t2;
@@ -652,10 +674,10 @@ struct WaveAttn {
                     t2 = vv[cb][1];
                 } else {
                     const int d1 = 16 * cb + l8, d2 = d1 + 8;
-                    t1 = load_lines16(vbase + (size_t)(d1 < hd ? d1 : 0) * bs + 8 * lh);
-                    t2 = load_lines16(vbase + (size_t)(d2 < hd ? d2 : 0) * bs + 8 * lh);
+                    t1 = load_lines16(vbase + (size_t)(d1 < vd ? d1 : 0) * bs + 8 * lh);
+                    t2 = load_lines16(vbase + (size_t)(d2 < vd ? d2 : 0) * bs + 8 * lh);
                 }
-                const uint32_t ok = vmask & opaque_mask(16 * cb + li < hd);
+                const uint32_t ok = vmask & opaque_mask(16 * cb + li < vd);
                 v0 = and_mask(swap_halves<0xC>(t1, t2), ok);
                 v1 = and_mask(swap_halves<0x3>(t2, t1), ok);
             }
@@ -692,7 +714,8 @@ __global__ __launch_bounds__(64) void attn_mfma_tile_kernel(AttnArgs a) {
     const PageLookup pl = {bt, nullptr, 0, 0};
     const KeySpan span = {kv_begin, kv_end, a.keep_first};
     const TileWalk walk = tile_walk(span);
-    for (int ti = 0; ti < walk.n; ++ti) w.tile(a, pl, kvh, walk.start(ti), span, lo, hi);
+    const float slope = a.slopes ? a.slopes[h] : 0.f;
+    for (int ti = 0; ti < walk.n; ++ti) w.tile(a, pl, kvh, walk.start(ti), span, lo, hi, slope, hi);
     const float fin = li < n ? finish_row<true>(a, h, w.m, w.l) : 0.f;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -702,7 +725,7 @@ __global__ __launch_bounds__(64) void attn_mfma_tile_kernel(AttnArgs a) {
 #pragma unroll
             for (int cb = 0; cb < WaveAttn<HD>::CB; ++cb) {
                 const int d = 16 * cb + li;
-                if (d < hd) store_out<bf16>(a, tok0 + row, h, d, w.o[cb][r] * fr);
+                if (d < a.vd) store_out<bf16>(a, tok0 + row, h, d, w.o[cb][r] * fr);
             }
         }
     }
@@ -764,7 +787,8 @@ __global__ __launch_bounds__(MAX_THREADS) void attn_mfma_decode_block_kernel(Att
         const KeySpan span = {kv_begin, kv_end, split == 0 ? min(a.keep_first, kv_begin) : 0};
         const TileWalk walk = tile_walk(span);
         const int lo = row_ok ? kv_begin : 1, hi = row_ok ? kv_end - 1 : 0;
-        for (int ti = wave; ti < walk.n; ti += n_waves) w.tile(a, pl, kvh, walk.start(ti), span, lo, hi);
+        const float slope = (a.slopes && row_ok) ? a.slopes[h0 + li] : 0.f;      // (a row is a query head here)
+        for (int ti = wave; ti < walk.n; ti += n_waves) w.tile(a, pl, kvh, walk.start(ti), span, lo, hi, slope, p);
     }
     const int stride = HD + 2;
     float* mine = wave_out + (size_t)wave * n * stride;
@@ -781,8 +805,9 @@ __global__ __launch_bounds__(MAX_THREADS) void attn_mfma_decode_block_kernel(Att
         }
     }
     __syncthreads();
-    for (int idx = threadIdx.x; idx < n * hd; idx += blockDim.x) {
-        const int row = idx / hd, d = idx - row * hd;
+    const int vd = a.vd;
+    for (int idx = threadIdx.x; idx < n * vd; idx += blockDim.x) {
+        const int row = idx / vd, d = idx - row * vd;
         float m = NEG_INF;
         for (int u = 0; u < n_waves; ++u) m = fmaxf(m, wave_out[((size_t)u * n + row) * stride + HD]);
         float l = 0.f, o = 0.f;
@@ -796,7 +821,7 @@ __global__ __launch_bounds__(MAX_THREADS) void attn_mfma_decode_block_kernel(Att
         if (a.splits == 1) {
             store_out<bf16>(a, tok, h, d, o * finish_row<true>(a, h, m, l));
         } else {
-            a.part_o[(((size_t)item * a.nh + h) * a.splits + split) * hd + d] = o;
+            a.part_o[(((size_t)item * a.nh + h) * a.splits + split) * vd + d] = o;
             if (d == 0) {
                 float* pml = a.part_ml + (((size_t)item * a.nh + h) * a.splits + split) * 2;
                 pml[0] = m == NEG_INF ? NEG_INF : m * LN2;
@@ -855,7 +880,9 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
             w_lo_max = first_visible(a, w_hi);
         }
     }
-    const float c2 = a.scale * LOG2E;
+    const bool shaped = shapes_scores(a);
+    const float slope = a.slopes ? a.slopes[h] : 0.f;
+    const float cs = shaped ? LOG2E : a.scale * LOG2E;
     float m = NEG_INF, l = 0.f;
     f32x4_t o[CB];
     bf16x8_t qf[KS];
@@ -957,8 +984,9 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
         // tiles that every row of this wave sees whole need no mask
         const bool whole = kt0 >= w_lo_max && kt0 + 63 <= w_hi_min && kt0 >= kv_begin;
         uint4 p_lo, p_hi;
-        const float alpha = whole ? softmax_step<false>(sc, kt0 + 16 * g, lo, hi, c2, m, l, p_lo, p_hi)
-                                  : softmax_step<true>(sc, kt0 + 16 * g, lo, hi, c2, m, l, p_lo, p_hi, span.keep);
+        if (shaped) shape_scores(sc, kt0 + 16 * g, a, slope, hi);
+        const float alpha = whole ? softmax_step<false>(sc, kt0 + 16 * g, lo, hi, cs, m, l, p_lo, p_hi)
+                                  : softmax_step<true>(sc, kt0 + 16 * g, lo, hi, cs, m, l, p_lo, p_hi, span.keep);
         const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0;
         float al[4] = {1.f, 1.f, 1.f, 1.f};
         if (rescale) {
@@ -1053,7 +1081,9 @@ __global__ __launch_bounds__(W * G * 64, W / 2) void attn_mfma_direct_kernel(Att
             w_lo_max = first_visible(a, w_hi);
         }
     }
-    const float c2 = a.scale * LOG2E;
+    const bool shaped = shapes_scores(a);
+    const float slope = a.slopes ? a.slopes[h] : 0.f;
+    const float cs = shaped ? LOG2E : a.scale * LOG2E;
     float m = NEG_INF, l = 0.f;
     f32x4_t o[CB];
     bf16x8_t qf[KS];
@@ -1145,8 +1175,9 @@ __global__ __launch_bounds__(W * G * 64, W / 2) void attn_mfma_direct_kernel(Att
         }
         const bool whole = kt0 >= w_lo_max && kt0 + 63 <= w_hi_min && kt0 >= kv_begin;
         uint4 p_lo, p_hi;
-        const float alpha = whole ? softmax_step<false>(sc, kt0 + 16 * g, lo, hi, c2, m, l, p_lo, p_hi)
-                                  : softmax_step<true>(sc, kt0 + 16 * g, lo, hi, c2, m, l, p_lo, p_hi, span.keep);
+        if (shaped) shape_scores(sc, kt0 + 16 * g, a, slope, hi);
+        const float alpha = whole ? softmax_step<false>(sc, kt0 + 16 * g, lo, hi, cs, m, l, p_lo, p_hi)
+                                  : softmax_step<true>(sc, kt0 + 16 * g, lo, hi, cs, m, l, p_lo, p_hi, span.keep);
         const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0;
         float al[4] = {1.f, 1.f, 1.f, 1.f};
         if (rescale) {
@@ -1208,8 +1239,10 @@ FX_API int fx_debug_set(const char* key, int value) {
     return 1;
 }
 
+// (value heads narrower than key heads, vd < hd in multiples of 16, run on the kernels in which a wave fetches its own
+// operands: attn_mfma_tile_kernel and attn_mfma_decode_block_kernel)
 static bool mfma_ok(int dtype, int hd, int bs, const void* q, long ldq, const void* k_pages, const void* v_pages, int vd = 0) {
-    return (vd == 0 || vd == hd) && dtype == FX_BF16 && hd % 16 == 0 && bs % 16 == 0 && hd % 8 == 0 && ldq % 8 == 0 &&
+    return (vd == 0 || vd == hd || (vd < hd && vd % 16 == 0)) && dtype == FX_BF16 && hd % 16 == 0 && bs % 16 == 0 && hd % 8 == 0 && ldq % 8 == 0 &&
            (((uintptr_t)q | (uintptr_t)k_pages | (uintptr_t)v_pages) % 16 == 0);
 }
 
@@ -1268,7 +1301,11 @@ FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void*
     const bool two_groups = g_groups ? g_groups == 2 : (long)n_items * nh <= fx_compute_units();
     if (dtype == FX_F32)
         attn_tile_kernel<float><<<grid, 64, 0, s>>>(a);
-    else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages, vd) && !shapes_scores(a)) {
+    else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages, vd) && vd != hd) {
+        if (hd <= 64) attn_mfma_tile_kernel<64><<<grid, 64, 0, s>>>(a);
+        else if (hd <= 128) attn_mfma_tile_kernel<128><<<grid, 64, 0, s>>>(a);
+        else attn_mfma_tile_kernel<256><<<grid, 64, 0, s>>>(a);
+    } else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages, vd)) {
         if (tile_q == 128 && hd == 128 && two_groups) attn_mfma_direct_kernel<128, 2, 8, 2><<<grid_blocks, 1024, 0, s>>>(a);
         else if (tile_q == 128 && hd == 64 && two_groups) attn_mfma_direct_kernel<64, 2, 8, 2><<<grid_blocks, 1024, 0, s>>>(a);
         else if (tile_q == 128 && hd == 128) attn_mfma_direct_kernel<128, 2, 8><<<grid_blocks, 512, 0, s>>>(a);
@@ -1313,7 +1350,7 @@ static int attn_decode_launch(void* stream, int dtype, const void* q, long ldq, 
     if (dtype == FX_F32) {
         attn_decode_kernel<float><<<grid, 64, 0, s>>>(a);
         attn_decode_merge_kernel<float><<<grid2, 128, splits * sizeof(float), s>>>(a);
-    } else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages, vd) && !shapes_scores(a)) {
+    } else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages, vd)) {
         const int group = nh / nkv;
         dim3 gridm(nkv * ((group + 15) / 16), n_items, splits);
         // as many waves per block (up to 8, and no more than a split has tiles) as their results fit in LDS

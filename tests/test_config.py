@@ -80,7 +80,8 @@ def test_stop_ids_are_one_or_several():
 
 
 def test_registry_is_closed(tmp_path):
-    assert known_architectures() == ["Kovalorn", "Qwen2MoeForCausalLM", "Rafilix"]
+    assert known_architectures() == ["Fokinex", "Kovalorn", "Qwen2MoeForCausalLM", "Rafilix"]
+    assert resolve({"architecture": "Fokinex"}).model_type == "fokinex"
     assert resolve({"architecture": "Rafilix"}).model_type == "rafilix"
     assert resolve({"architecture": "Kovalorn"}).model_type == "kovalorn"
     with pytest.raises(ConfigError) as e:
