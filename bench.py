@@ -405,13 +405,15 @@ def run_workload(name: str, args) -> int:
     return 0
 
 
-# ---- Rafilix and Kovalorn beside the closest existing model, at equal layer sizes ----------------------------------
+# ---- Rafilix, Kovalorn and Fokinex beside the closest existing model, at equal layer sizes ----------------------------------
 # Layer sizes that resemble a real model's; every model is four layers of random weights.  The Rafilix layers are
 # measured by kind (all attention, all recurrent) and in the design's usual mixture, the Qwen2-MoE layers have the
 # same width, heads, experts and expert width and no shared expert (Rafilix has none).
 DESIGN_SIZES = {
-    "1k": dict(width=1024, heads=8, kv_heads=2, dim=128, experts=16, identity=2, top=2, ff=704, vocab=32000),
-    "2k": dict(width=2048, heads=16, kv_heads=4, dim=128, experts=60, identity=4, top=4, ff=1408, vocab=32000),
+    "1k": dict(width=1024, heads=8, kv_heads=2, dim=128, experts=16, identity=2, top=2, ff=704, vocab=32000, dense_ff=2816,
+               q_rank=384, kv_rank=192, rot_dim=64),
+    "2k": dict(width=2048, heads=16, kv_heads=4, dim=128, experts=60, identity=4, top=4, ff=1408, vocab=32000, dense_ff=5632,
+               q_rank=768, kv_rank=192, rot_dim=64),
 }
 
 
@@ -447,10 +449,43 @@ def design_configs(s: dict) -> dict:
             layers.append({"type": "attention", "mixer": mixer, "mlp": kmlp})
         return {"architecture": "Kovalorn", "vocab": s["vocab"], "width": s["width"], "norm": {"eps": 1e-5}, "logit_scale": 1.0,
                 "layers": layers, "max_positions": 16384}
+    # Fokinex: layers whose two sublayers read one norm; latent attention (a latent and a rotated key part of 256
+    # numbers a position together, the most the attention kernels take as one key head) under a window with sinks, or
+    # capped attention beside a delta rule with one decay per head; dense feed-forwards.  Beside it Kovalorn layers
+    # with the same dense feed-forward, and (above) Rafilix's delta-rule layers.
+    def fokinex(kinds):
+        dense = {"kind": "dense", "ff": s["dense_ff"]}
+        layers = []
+        for i, kind in enumerate(kinds):
+            if kind == "parallel":
+                mixer = {"left": {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": s["dim"], "vdim": s["dim"],
+                                  "scale": s["dim"] ** -0.5, "softcap": 30.0, "mask": {"size": 8192}},
+                         "right": {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": s["dim"], "vdim": s["dim"], "conv": 4},
+                         "left_scale": 1.0, "right_scale": 1.0}
+            else:
+                mixer = {"heads": s["heads"], "dim": s["dim"], "rot_dim": s["rot_dim"], "vdim": s["dim"], "q_rank": s["q_rank"],
+                         "kv_rank": s["kv_rank"], "scale": (s["dim"] + s["rot_dim"]) ** -0.5, "mask": {"size": 8192},
+                         "rot": {"base": 10000.0, "dims": s["rot_dim"],
+                                 "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+                if kind == "reader":
+                    mixer["kv_from"] = 1
+            layers.append({"type": "parallel" if kind == "parallel" else "latent_attention", "mixer": mixer, "mlp": dense})
+        return {"architecture": "Fokinex", "vocab": s["vocab"], "width": s["width"], "norm": {"eps": 1e-5},
+                "embedding": {"scale": s["width"] ** 0.5}, "layers": layers, "max_positions": 16384}
+
+    def kovalorn_dense():
+        mixer = {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": s["dim"], "vdim": s["dim"], "scale": s["dim"] ** -0.5,
+                 "mask": {"size": 8192, "keep_first": 64}}
+        return {"architecture": "Kovalorn", "vocab": s["vocab"], "width": s["width"], "norm": {"eps": 1e-5}, "logit_scale": 1.0,
+                "layers": [{"type": "attention", "mixer": mixer, "mlp": {"kind": "dense", "ff": s["dense_ff"]}}] * 4,
+                "max_positions": 16384}
+    more = {"kovalorn dense": kovalorn_dense(), "fokinex latent": fokinex(["latent"] * 4),
+            "fokinex side by side": fokinex(["parallel"] * 4),
+            "fokinex mixed": fokinex(["latent", "latent", "reader", "parallel"])}
     return {"qwen2-moe": qwen, "rafilix attention": rafilix([attn] * 4), "rafilix recurrent": rafilix([delta] * 4),
             "rafilix mixed": rafilix([attn, delta, delta, attn]),
             "qwen2-moe shared expert": dict(qwen, shared_expert_intermediate_size=2 * s["ff"]),
-            "kovalorn": kovalorn(()), "kovalorn shared keys": kovalorn((2, 3))}
+            "kovalorn": kovalorn(()), "kovalorn shared keys": kovalorn((2, 3)), **more}
 
 
 def compare_designs(args) -> int:

@@ -652,6 +652,20 @@ struct WaveAttn {
                 sc[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ku), qf[u], sc[kb], 0, 0, 0);
             }
         }
+        // Heads too wide for their values to be fetched before the scores: the values arrive in groups of VG column
+        // blocks, a group's loads issued together and a group ahead of the products that use them (the first one before
+        // the softmax), so that a tile waits for memory CB / VG times and not once per column block.
+        constexpr int VG = CB < 4 ? CB : 4;
+        uint4 ahead[EARLY_V ? 1 : VG][2];
+        auto fetch_values = [&](int c0) {
+#pragma unroll
+            for (int j = 0; j < VG; ++j) {
+                const int d1 = 16 * (c0 + j) + l8, d2 = d1 + 8;
+                ahead[EARLY_V ? 0 : j][0] = load_lines16(vbase + (size_t)(d1 < vd ? d1 : 0) * bs + 8 * lh);
+                ahead[EARLY_V ? 0 : j][1] = load_lines16(vbase + (size_t)(d2 < vd ? d2 : 0) * bs + 8 * lh);
+            }
+        };
+        if (!EARLY_V) fetch_values(0);
         // softmax on this lane's 16 scores (keys kt0 + 16g + 4kb + r); the row's four lanes share max and sum
         uint4 p_lo, p_hi;
         const bool shaped = shapes_scores(a);
@@ -664,28 +678,31 @@ struct WaveAttn {
             for (int r = 0; r < 4; ++r) al[r] = __shfl(alpha, 4 * g + r, 64);
         }
 #pragma unroll
-        for (int cb = 0; cb < CB; ++cb) {
-            if (HD > 128 && 16 * cb >= vd) continue;              // (the same in every lane: columns past the value head's size)
-            uint4 v0, v1;
-            {
-                uint4 t1, t2;
-                if (EARLY_V) {
-                    t1 = vv[cb][0];
-                    t2 = vv[cb][1];
-                } else {
-                    const int d1 = 16 * cb + l8, d2 = d1 + 8;
-                    t1 = load_lines16(vbase + (size_t)(d1 < vd ? d1 : 0) * bs + 8 * lh);
-                    t2 = load_lines16(vbase + (size_t)(d2 < vd ? d2 : 0) * bs + 8 * lh);
+        for (int c0 = 0; c0 < CB; c0 += VG) {
+            if (HD > 128 && 16 * c0 >= vd) break;                 // (the same in every lane: columns past the value head's size)
+            uint4 now[EARLY_V ? 1 : VG][2];
+            if (!EARLY_V) {
+#pragma unroll
+                for (int j = 0; j < VG; ++j) {
+                    now[j][0] = ahead[j][0];
+                    now[j][1] = ahead[j][1];
                 }
+                if (c0 + VG < CB && 16 * (c0 + VG) < vd) fetch_values(c0 + VG);
+            }
+#pragma unroll
+            for (int j = 0; j < VG; ++j) {
+                const int cb = c0 + j;
+                const uint4 t1 = EARLY_V ? vv[EARLY_V ? cb : 0][0] : now[EARLY_V ? 0 : j][0];
+                const uint4 t2 = EARLY_V ? vv[EARLY_V ? cb : 0][1] : now[EARLY_V ? 0 : j][1];
                 const uint32_t ok = vmask & opaque_mask(16 * cb + li < vd);
-                v0 = and_mask(swap_halves<0xC>(t1, t2), ok);
-                v1 = and_mask(swap_halves<0x3>(t2, t1), ok);
+                uint4 v0 = and_mask(swap_halves<0xC>(t1, t2), ok);
+                uint4 v1 = and_mask(swap_halves<0x3>(t2, t1), ok);
+                if (edge) {
+                    v0 = keep_keys(v0, kg, span);
+                    v1 = keep_keys(v1, kg + 8, span);
+                }
+                o[cb] = pv_step(o[cb], rescale, al, p_lo, p_hi, v0, v1);
             }
-            if (edge) {
-                v0 = keep_keys(v0, kg, span);
-                v1 = keep_keys(v1, kg + 8, span);
-            }
-            o[cb] = pv_step(o[cb], rescale, al, p_lo, p_hi, v0, v1);
         }
     }
 };
@@ -857,7 +874,7 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
     const int kvh = h / (a.nh / a.nkv);
     const int tok_first = a.item_tok[item], n_all = a.item_n[item];
     const int* bt = a.block_table + (size_t)a.item_seq[item] * a.max_blocks;
-    const int hd = a.hd, bs = a.bs;
+    const int hd = a.hd, bs = a.bs, vd = a.vd;      // (vd <= hd: the value heads may be narrower than the key heads)
     const int pmin = a.positions[tok_first], pmax = a.positions[tok_first + n_all - 1];
     const int kv_begin = first_visible(a, pmin);
     const int kv_end = pmax + 1;
@@ -917,7 +934,7 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
             page_slot(a, live[j] ? key0 : safe_group, blk, slot);
             const size_t page = pl.page(blk);
             kbase[j] = ((page * a.nkv + kvh) * bs + slot) * hd;
-            vbase[j] = (page * a.nkv + kvh) * hd * bs + slot;
+            vbase[j] = (page * a.nkv + kvh) * vd * bs + slot;
         }
 #pragma unroll
         for (int i = 0; i < NK; ++i) {
@@ -935,8 +952,12 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
             const int c = tid + i * 256;
             if (c < VCH) {
                 const int d = c >> 3, k8 = (c & 7) * 8;
-                const bool ok = d < hd && live[k8 >> 4];
-                uint4 v = *(const uint4*)((const bf16*)a.v_pages + vbase[k8 >> 4] + (size_t)(d < hd ? d : 0) * bs + (k8 & 15));
+                if (HD > 128 && d >= vd) {       // (whole groups of 32 rows past the value head's size: nothing to load)
+                    vreg[i] = make_uint4(0, 0, 0, 0);
+                    continue;
+                }
+                const bool ok = d < vd && live[k8 >> 4];
+                uint4 v = *(const uint4*)((const bf16*)a.v_pages + vbase[k8 >> 4] + (size_t)(d < vd ? d : 0) * bs + (k8 & 15));
                 if (!span.holds_tile(kt0)) v = keep_keys(v, kt0 + k8, span);
                 vreg[i] = ok ? v : make_uint4(0, 0, 0, 0);
             }
@@ -977,6 +998,7 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
             sc[kb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int u = 0; u < KS; ++u) {
+                if (HD > 128 && 32 * u >= hd) continue;           // (the same in every lane: k-steps past the head's size)
                 const bf16x8_t kf = *(const bf16x8_t*)(Ks + (kb * 16 + li) * KROW + 32 * u + 8 * g);
                 sc[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[u], sc[kb], 0, 0, 0);
             }
@@ -995,6 +1017,7 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
         }
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) {
+            if (HD > 128 && 16 * cb >= vd) continue;              // (the same in every lane: columns past the value head's size)
             const bf16* vr = Vs + (16 * cb + li) * VROW + 16 * g;
             o[cb] = pv_step(o[cb], rescale, al, p_lo, p_hi, *(const uint4*)vr, *(const uint4*)(vr + 8));
         }
@@ -1008,7 +1031,7 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) {
                 const int d = 16 * cb + li;
-                if (d < hd) store_out<bf16>(a, tok0 + row, h, d, o[cb][r] * fr);
+                if (d < vd) store_out<bf16>(a, tok0 + row, h, d, o[cb][r] * fr);
             }
         }
     }
@@ -1301,10 +1324,12 @@ FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void*
     const bool two_groups = g_groups ? g_groups == 2 : (long)n_items * nh <= fx_compute_units();
     if (dtype == FX_F32)
         attn_tile_kernel<float><<<grid, 64, 0, s>>>(a);
-    else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages, vd) && vd != hd) {
+    else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages, vd) && hd > 128) {
+        // the widest heads: tiles of 64 keys (34 KB) and their values (36 KB) staged in LDS for the block's 64 queries
+        attn_mfma_block_kernel<256><<<grid_blocks, 256, 0, s>>>(a);
+    } else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages, vd) && vd != hd) {
         if (hd <= 64) attn_mfma_tile_kernel<64><<<grid, 64, 0, s>>>(a);
-        else if (hd <= 128) attn_mfma_tile_kernel<128><<<grid, 64, 0, s>>>(a);
-        else attn_mfma_tile_kernel<256><<<grid, 64, 0, s>>>(a);
+        else attn_mfma_tile_kernel<128><<<grid, 64, 0, s>>>(a);
     } else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages, vd)) {
         if (tile_q == 128 && hd == 128 && two_groups) attn_mfma_direct_kernel<128, 2, 8, 2><<<grid_blocks, 1024, 0, s>>>(a);
         else if (tile_q == 128 && hd == 64 && two_groups) attn_mfma_direct_kernel<64, 2, 8, 2><<<grid_blocks, 1024, 0, s>>>(a);
@@ -1318,7 +1343,7 @@ FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void*
         else if (hd <= 32) attn_mfma_block_kernel<32><<<grid_blocks, 256, 0, s>>>(a);
         else if (hd <= 64) attn_mfma_block_kernel<64><<<grid_blocks, 256, 0, s>>>(a);
         else if (hd <= 128) attn_mfma_block_kernel<128><<<grid_blocks, 256, 0, s>>>(a);
-        else attn_mfma_tile_kernel<256><<<grid, 64, 0, s>>>(a);       // too large to stage in LDS
+        else return fx_fail("attn_tiles: no kernel for a head size of %d", hd);
     } else
         attn_tile_kernel<bf16><<<grid, 64, 0, s>>>(a);
     FX_CHECK_LAUNCH("attn_tiles");

@@ -229,3 +229,13 @@ def test_a_cache_holds_what_its_widest_reader_sees():
     latent = model.blocks[0].mixer
     assert latent.page_shapes(16) == {"k": (1, 16, 40), "v": (1, 32, 16)}      # (c | rotated part) and c, one head
     assert model.blocks[2].mixer.page_shapes(16) == latent.page_shapes(16)
+
+
+def test_named_shape_of_the_design_reads():
+    from ferrox_amd.config import presets
+    raw = presets.load("fokinex-2k")
+    assert resolve(raw).name == "Fokinex"
+    cfg = FokinexConfig.from_dict(raw)
+    assert len(cfg.layers) == 8 and {layer.type for layer in cfg.layers} == {"latent_attention", "parallel"}
+    assert [layer.mixer.kv_from for layer in cfg.layers if layer.type == "latent_attention"] == [None, None, 1, None, None, 5]
+    assert Model(build_spec(cfg)).cache_groups() == {("window", 8192): 8192}

@@ -105,7 +105,8 @@ def attention_reference(q, k, v, scale, window, sinks, gate, softcap, slopes):
 @pytest.mark.parametrize("dtype,hd,vd,bs,G", [
     ("float32", 24, 24, 16, 2), ("bfloat16", 64, 64, 64, 2), ("bfloat16", 128, 128, 64, 1), ("bfloat16", 48, 48, 16, 2),
     ("bfloat16", 32, 32, 16, 4), ("bfloat16", 20, 20, 16, 2), ("bfloat16", 144, 128, 64, 1), ("bfloat16", 80, 64, 16, 1),
-    ("float32", 40, 32, 16, 1)])
+    ("float32", 40, 32, 16, 1), ("bfloat16", 256, 192, 64, 1), ("bfloat16", 160, 160, 16, 2), ("bfloat16", 256, 256, 16, 1),
+    ("bfloat16", 208, 64, 64, 1)])
 def test_attention_kernels_with_capped_scores_and_distance_slopes(dtype, hd, vd, bs, G):
     """The attention kernels alone with a cap on the scores, a penalty per head for distance, a sink and a gate, and
     with value heads narrower than key heads over one shared key head (what latent attention asks of them): a prompt
