@@ -854,7 +854,7 @@ __global__ __launch_bounds__(MAX_THREADS) void attn_mfma_decode_block_kernel(Att
 // transposed V once, and every wave takes its operands from there.  While a tile is multiplied
 // the next one is already on its way from memory into registers.
 template <int HD>
-__global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
+__global__ __launch_bounds__(256, HD > 128 ? 2 : 1) void attn_mfma_block_kernel(AttnArgs a) {
     constexpr int KS = HD / 32, CB = HD / 16;
     constexpr int KROW = HD + 8;          // bf16 elements per staged key row (16 bytes of padding)
     constexpr int VROW = 64 + 8;          // bf16 elements per staged value row
@@ -912,7 +912,10 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
         qf[u] = __builtin_bit_cast(bf16x8_t, v);
     }
 
-    uint4 kreg_a[NK], vreg_a[NV], kreg_b[NK], vreg_b[NV];     // two tiles on their way from memory
+    // Two tiles on their way from memory; the widest heads keep one (DEEP false): their registers then allow two blocks
+    // on a CU, whose waves fill each other's waits, and a tile's products take longer than its loads.
+    constexpr bool DEEP = HD <= 128;
+    uint4 kreg_a[NK], vreg_a[NV], kreg_b[DEEP ? NK : 1], vreg_b[DEEP ? NV : 1];
     // Loads are issued without branches: a key outside [kv_begin, kv_end) (its page may have been
     // given back) reads from a group of keys that is inside, and its data is replaced by zeros.
     const int safe_group = (kv_end - 1) & ~15;
@@ -981,15 +984,19 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
     };
 
     fetch(kreg_a, vreg_a, walk.start(0));
-    if (1 < walk.n) fetch(kreg_b, vreg_b, walk.start(1));
+    if (DEEP && 1 < walk.n) fetch(kreg_b, vreg_b, walk.start(1));
     int parity = 0;
     for (int ti = 0; ti < walk.n; ++ti, parity ^= 1) {
         const int kt0 = walk.start(ti);
         lds_barrier();            // the previous tile has been read by every wave
-        if (parity == 0) stage(kreg_a, vreg_a); else stage(kreg_b, vreg_b);
+        if (!DEEP || parity == 0) stage(kreg_a, vreg_a); else stage(kreg_b, vreg_b);
         lds_barrier();
-        if (ti + 2 < walk.n) {     // the registers just emptied take the tile after the next
-            if (parity == 0) fetch(kreg_a, vreg_a, walk.start(ti + 2)); else fetch(kreg_b, vreg_b, walk.start(ti + 2));
+        if (DEEP) {
+            if (ti + 2 < walk.n) {     // the registers just emptied take the tile after the next
+                if (parity == 0) fetch(kreg_a, vreg_a, walk.start(ti + 2)); else fetch(kreg_b, vreg_b, walk.start(ti + 2));
+            }
+        } else if (ti + 1 < walk.n) {
+            fetch(kreg_a, vreg_a, walk.start(ti + 1));
         }
         if (kt0 > w_hi || (kt0 + 64 <= w_lo && kt0 >= span.keep)) continue;      // nothing in this tile for this wave's rows
         f32x4_t sc[4];
