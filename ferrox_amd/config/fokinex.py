@@ -93,8 +93,8 @@ def _latent(r: ConfigReader, index: int) -> LatentAttentionConfig:
     heads, dim = r.integer("heads", minimum=1), r.integer("dim", minimum=1)
     rot_dim, vdim = r.integer("rot_dim", minimum=0), r.integer("vdim", minimum=1)
     q_rank, kv_rank = r.integer("q_rank", minimum=1), r.integer("kv_rank", minimum=1)
-    if kv_rank + rot_dim > limits.HEAD_DIM_MAX:
-        raise ConfigError(f"{r.where}: kv_rank {kv_rank} + rot_dim {rot_dim} is more than the attention kernels' {limits.HEAD_DIM_MAX}")
+    if kv_rank + rot_dim > limits.HEAD_DIM_MAX_ANY:
+        raise ConfigError(f"{r.where}: kv_rank {kv_rank} + rot_dim {rot_dim} is more than the attention kernels' {limits.HEAD_DIM_MAX_ANY}")
     rot = None
     rr = _section(r, "rot", required=False)
     if rr is not None:

@@ -19,7 +19,8 @@
 
 FX_DEFINE_LAST_ERROR()
 
-#define HD_MAX 256
+#define HD_MAX 256          // the widest head of the matrix-unit kernels
+#define HD_MAX_ANY 512      // the widest head of the kernels for any shape (float32, or bfloat16 heads beyond HD_MAX)
 #define TQ 16
 #define NEG_INF (-INFINITY)
 
@@ -173,9 +174,10 @@ __device__ __forceinline__ const T* value_col(const AttnArgs& a, const int* bt, 
 // queries of one sequence; one wave per (quarter of an item = up to 16 queries,
 // head); lanes are keys for the scores and head dimensions for the output.
 // ---------------------------------------------------------------------------
-template <typename T>
+// HDM: the widest head this instance takes (its queries in LDS and its outputs in registers are sized by it).
+template <typename T, int HDM = HD_MAX>
 __global__ __launch_bounds__(64) void attn_tile_kernel(AttnArgs a) {
-    __shared__ float Qs[TQ][HD_MAX];
+    __shared__ float Qs[TQ][HDM];
     __shared__ float Ps[TQ][64];
     const int item = blockIdx.x >> 2, sub = blockIdx.x & 3, h = blockIdx.y, lane = threadIdx.x;
     const int kvh = h / (a.nh / a.nkv);
@@ -199,13 +201,13 @@ __global__ __launch_bounds__(64) void attn_tile_kernel(AttnArgs a) {
     const bool shaped = shapes_scores(a);
     const float slope = a.slopes ? a.slopes[h] : 0.f;
 
-    float m[TQ], l[TQ], o[HD_MAX / 64][TQ];
+    float m[TQ], l[TQ], o[HDM / 64][TQ];
 #pragma unroll
     for (int i = 0; i < TQ; ++i) {
         m[i] = NEG_INF;
         l[i] = 0.f;
 #pragma unroll
-        for (int dd = 0; dd < HD_MAX / 64; ++dd) o[dd][i] = 0.f;
+        for (int dd = 0; dd < HDM / 64; ++dd) o[dd][i] = 0.f;
     }
     __syncthreads();
 
@@ -239,7 +241,7 @@ __global__ __launch_bounds__(64) void attn_tile_kernel(AttnArgs a) {
         }
         __syncthreads();
 #pragma unroll
-        for (int dd = 0; dd < HD_MAX / 64; ++dd) {
+        for (int dd = 0; dd < HDM / 64; ++dd) {
             const int d = dd * 64 + lane;
             if (d < a.vd) {
 #pragma unroll
@@ -256,7 +258,7 @@ __global__ __launch_bounds__(64) void attn_tile_kernel(AttnArgs a) {
         __syncthreads();
     }
 #pragma unroll
-    for (int dd = 0; dd < HD_MAX / 64; ++dd) {
+    for (int dd = 0; dd < HDM / 64; ++dd) {
         const int d = dd * 64 + lane;
         if (d < a.vd) {
 #pragma unroll
@@ -271,9 +273,9 @@ __global__ __launch_bounds__(64) void attn_tile_kernel(AttnArgs a) {
 // `chunk` positions; one wave per (sequence, head, chunk) writes a partial
 // (max, sum, output), and a second kernel merges the chunks in ascending order.
 // ---------------------------------------------------------------------------
-template <typename T>
+template <typename T, int HDM = HD_MAX>
 __global__ __launch_bounds__(64) void attn_decode_kernel(AttnArgs a) {
-    __shared__ float Qs[HD_MAX];
+    __shared__ float Qs[HDM];
     __shared__ float Ps[64];
     const int item = blockIdx.x, h = blockIdx.y, split = blockIdx.z, lane = threadIdx.x;
     const int kvh = h / (a.nh / a.nkv);
@@ -297,9 +299,9 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(AttnArgs a) {
     }
     for (int d = lane; d < hd; d += 64) Qs[d] = to_float(((const T*)a.q)[(size_t)tok * a.ldq + (size_t)h * hd + d]) * a.scale;
     __syncthreads();
-    float m = NEG_INF, l = 0.f, o[HD_MAX / 64];
+    float m = NEG_INF, l = 0.f, o[HDM / 64];
 #pragma unroll
-    for (int dd = 0; dd < HD_MAX / 64; ++dd) o[dd] = 0.f;
+    for (int dd = 0; dd < HDM / 64; ++dd) o[dd] = 0.f;
     for (int kt0 = s0; kt0 < kv_end; kt0 += 64) {
         if (!span.touches(kt0, 64)) continue;      // a tile between the kept keys and the window
         const int t = kt0 + lane;
@@ -319,7 +321,7 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(AttnArgs a) {
         Ps[lane] = pr;
         __syncthreads();
 #pragma unroll
-        for (int dd = 0; dd < HD_MAX / 64; ++dd) {
+        for (int dd = 0; dd < HDM / 64; ++dd) {
             const int d = dd * 64 + lane;
             if (d < a.vd) {
                 float acc = o[dd] * al;
@@ -334,7 +336,7 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(AttnArgs a) {
         __syncthreads();
     }
 #pragma unroll
-    for (int dd = 0; dd < HD_MAX / 64; ++dd) {
+    for (int dd = 0; dd < HDM / 64; ++dd) {
         const int d = dd * 64 + lane;
         if (d < a.vd) po[d] = o[dd];
     }
@@ -1272,7 +1274,7 @@ FX_API int fx_debug_set(const char* key, int value) {
 // (value heads narrower than key heads, vd < hd in multiples of 16, run on the kernels in which a wave fetches its own
 // operands: attn_mfma_tile_kernel and attn_mfma_decode_block_kernel)
 static bool mfma_ok(int dtype, int hd, int bs, const void* q, long ldq, const void* k_pages, const void* v_pages, int vd = 0) {
-    return (vd == 0 || vd == hd || (vd < hd && vd % 16 == 0)) && dtype == FX_BF16 && hd % 16 == 0 && bs % 16 == 0 && hd % 8 == 0 && ldq % 8 == 0 &&
+    return hd <= HD_MAX && (vd == 0 || vd == hd || (vd < hd && vd % 16 == 0)) && dtype == FX_BF16 && hd % 16 == 0 && bs % 16 == 0 && hd % 8 == 0 && ldq % 8 == 0 &&
            (((uintptr_t)q | (uintptr_t)k_pages | (uintptr_t)v_pages) % 16 == 0);
 }
 
@@ -1280,14 +1282,14 @@ static bool mfma_ok(int dtype, int hd, int bs, const void* q, long ldq, const vo
 static int check_common(const char* who, int dtype, int nh, int nkv, int hd, int bs, int window, float scale, int vd = 0, int mask_chunk = 0,
                         int keep_first = 0) {
     FX_REQUIRE(keep_first >= 0 && !(keep_first > 0 && mask_chunk > 0), "%s: kept first keys (%d) go with a window, not with a chunked mask (%d)", who, keep_first, mask_chunk);
-    FX_REQUIRE(vd >= 0 && vd <= HD_MAX, "%s: value head size %d is outside 1..%d", who, vd, HD_MAX);
+    FX_REQUIRE(vd >= 0 && vd <= HD_MAX_ANY, "%s: value head size %d is outside 1..%d", who, vd, HD_MAX_ANY);
     FX_REQUIRE(mask_chunk >= 0 && !(mask_chunk > 0 && window > 0), "%s: a window (%d) or a chunked mask (%d), not both", who, window, mask_chunk);
     // (the bfloat16 kernels take a row's maximum over the raw scores and scale it once, which is the maximum of
     // the scaled scores only under a positive scale)
     FX_REQUIRE(scale > 0.f && scale < INFINITY, "%s: the scale of the scores must be positive and finite, got %g", who, (double)scale);
     FX_REQUIRE(dtype == FX_F32 || dtype == FX_BF16, "%s: unknown dtype %d", who, dtype);
     FX_REQUIRE(nh > 0 && nkv > 0 && nh % nkv == 0, "%s: n_heads %d must be a multiple of n_kv_heads %d", who, nh, nkv);
-    FX_REQUIRE(hd > 0 && hd <= HD_MAX, "%s: head_dim %d is outside 1..%d", who, hd, HD_MAX);
+    FX_REQUIRE(hd > 0 && hd <= HD_MAX_ANY, "%s: head_dim %d is outside 1..%d", who, hd, HD_MAX_ANY);
     FX_REQUIRE(bs > 0, "%s: block size %d", who, bs);
     FX_REQUIRE(window >= 0, "%s: window %d", who, window);
     return 0;
@@ -1329,8 +1331,13 @@ FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void*
     // (measured: 512-token portions at depth 8k-24k 130 and 360 us against 214 and 616 us; from 448 blocks on, one
     // group and two blocks to a CU are as fast or faster)
     const bool two_groups = g_groups ? g_groups == 2 : (long)n_items * nh <= fx_compute_units();
-    if (dtype == FX_F32)
+    const bool beyond = hd > HD_MAX || vd > HD_MAX;      // heads wider than the matrix-unit kernels take
+    if (dtype == FX_F32 && beyond)
+        attn_tile_kernel<float, HD_MAX_ANY><<<grid, 64, 0, s>>>(a);
+    else if (dtype == FX_F32)
         attn_tile_kernel<float><<<grid, 64, 0, s>>>(a);
+    else if (beyond)
+        attn_tile_kernel<bf16, HD_MAX_ANY><<<grid, 64, 0, s>>>(a);
     else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages, vd) && hd > 128) {
         // the widest heads: tiles of 64 keys (34 KB) and their values (36 KB) staged in LDS for the block's 64 queries
         attn_mfma_block_kernel<256><<<grid_blocks, 256, 0, s>>>(a);
@@ -1379,9 +1386,14 @@ static int attn_decode_launch(void* stream, int dtype, const void* q, long ldq, 
     a.part_o = part_o; a.part_ml = part_ml; a.splits = splits; a.chunk = chunk;
     dim3 grid(n_items, nh, splits), grid2(n_items, nh);
     hipStream_t s = (hipStream_t)stream;
+    const bool beyond = hd > HD_MAX || vd > HD_MAX;      // heads wider than the matrix-unit kernels take
     if (dtype == FX_F32) {
-        attn_decode_kernel<float><<<grid, 64, 0, s>>>(a);
+        if (beyond) attn_decode_kernel<float, HD_MAX_ANY><<<grid, 64, 0, s>>>(a);
+        else attn_decode_kernel<float><<<grid, 64, 0, s>>>(a);
         attn_decode_merge_kernel<float><<<grid2, 128, splits * sizeof(float), s>>>(a);
+    } else if (beyond) {
+        attn_decode_kernel<bf16, HD_MAX_ANY><<<grid, 64, 0, s>>>(a);
+        attn_decode_merge_kernel<bf16><<<grid2, 128, splits * sizeof(float), s>>>(a);
     } else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages, vd)) {
         const int group = nh / nkv;
         dim3 gridm(nkv * ((group + 15) / 16), n_items, splits);

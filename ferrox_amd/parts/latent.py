@@ -67,9 +67,10 @@ class LatentAttention(Mixer):
         if min(self.n_heads, self.head_dim, self.v_dim, self.q_rank, self.kv_rank) < 1 or self.rot_dim < 0:
             raise ValueError("latent attention: heads, sizes and ranks are positive")
         self.key_width = self.kv_rank + self.rot_dim          # what the attention kernels see as the one key head
-        if self.key_width > limits.HEAD_DIM_MAX:
+        # (up to HEAD_DIM_MAX on the matrix units; wider, on the kernels for any shape)
+        if self.key_width > limits.HEAD_DIM_MAX_ANY:
             raise ValueError(f"latent attention: kv_rank {kv_rank} + rot_dim {rot_dim} is more than the attention kernels' "
-                             f"{limits.HEAD_DIM_MAX}")
+                             f"{limits.HEAD_DIM_MAX_ANY}")
         self.scale = float(scale)
         if not 0.0 < self.scale < math.inf:
             raise ValueError(f"the scale of the attention scores must be positive and finite, got {self.scale}")

@@ -193,7 +193,7 @@ def test_configuration_reads_every_size_from_the_file():
     (lambda c: c["layers"][4]["mixer"].update(kv_from=2), "no latents of its own"),
     (lambda c: c["layers"][2]["mixer"].update(kv_rank=16), "another latent size"),
     (lambda c: c["layers"][0]["mixer"]["rot"].update(dims=10), "at most rot_dim"),
-    (lambda c: c["layers"][0]["mixer"].update(kv_rank=300), "attention kernels"),
+    (lambda c: c["layers"][0]["mixer"].update(kv_rank=510), "attention kernels"),
     (lambda c: c["layers"][1]["mixer"]["left"].update(vdim=8), "keys are the values"),
     (lambda c: c["layers"][1]["mixer"]["left"].update(kv_heads=3), "not a multiple"),
     (lambda c: c["layers"][1]["mixer"]["right"].update(conv=40), "taps"),

@@ -54,6 +54,8 @@ SINGLE = {
     "latent_no_rotated_part": u.config([u.latent_layer(heads=2, dim=16, rot_dim=0, vdim=8, q_rank=8, kv_rank=16, window=15)]),
     "latent_shared": u.config([u.latent_layer(heads=4, dim=8, rot_dim=8, vdim=16, q_rank=12, kv_rank=24, window=12, mlp=u.dense(24)),
                                u.latent_layer(heads=2, dim=16, rot_dim=8, vdim=8, q_rank=20, kv_rank=24, window=30, kv_from=0)]),
+    "latent_wide": u.config([u.latent_layer(heads=3, dim=16, rot_dim=32, vdim=24, q_rank=24, kv_rank=272, window=19, scale=0.4, mlp=u.dense(32)),
+                             u.latent_layer(heads=2, dim=8, rot_dim=32, vdim=16, q_rank=16, kv_rank=272, window=40, scale=0.4, kv_from=0)]),
     "latent_one_head": u.config([u.latent_layer(heads=1, dim=32, rot_dim=4, vdim=32, q_rank=16, kv_rank=24, window=5, scale=0.3)]),
     "left_alone": u.config([u.parallel_layer(heads=4, kv_heads=2, dim=16, window=9, scale=0.5, softcap=3.0, left_scale=1.3, right_scale=0.0)]),
     "left_no_cap_no_mask": u.config([u.parallel_layer(heads=3, kv_heads=3, dim=8, window=0, scale=0.8, softcap=None, left_scale=1.0, right_scale=0.0)]),
@@ -106,7 +108,7 @@ def attention_reference(q, k, v, scale, window, sinks, gate, softcap, slopes):
     ("float32", 24, 24, 16, 2), ("bfloat16", 64, 64, 64, 2), ("bfloat16", 128, 128, 64, 1), ("bfloat16", 48, 48, 16, 2),
     ("bfloat16", 32, 32, 16, 4), ("bfloat16", 20, 20, 16, 2), ("bfloat16", 144, 128, 64, 1), ("bfloat16", 80, 64, 16, 1),
     ("float32", 40, 32, 16, 1), ("bfloat16", 256, 192, 64, 1), ("bfloat16", 160, 160, 16, 2), ("bfloat16", 256, 256, 16, 1),
-    ("bfloat16", 208, 64, 64, 1)])
+    ("bfloat16", 208, 64, 64, 1), ("bfloat16", 288, 256, 16, 1), ("float32", 320, 272, 64, 1)])
 def test_attention_kernels_with_capped_scores_and_distance_slopes(dtype, hd, vd, bs, G):
     """The attention kernels alone with a cap on the scores, a penalty per head for distance, a sink and a gate, and
     with value heads narrower than key heads over one shared key head (what latent attention asks of them): a prompt
