@@ -809,6 +809,38 @@ __global__ __launch_bounds__(MAX_THREADS) void attn_mfma_decode_block_kernel(Att
         const float slope = (a.slopes && row_ok) ? a.slopes[h0 + li] : 0.f;      // (a row is a query head here)
         for (int ti = wave; ti < walk.n; ti += n_waves) w.tile(a, pl, kvh, walk.start(ti), span, lo, hi, slope, p);
     }
+    if (n_waves == 1) {
+        // one wave: nothing to merge, the rows go out from the registers that hold them (lane (li, g) has rows
+        // 4g .. 4g + 3 of columns 16 cb + li; a row's maximum and sum sit in the lanes whose li is the row)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int row = 4 * g + r;
+            const float m = __shfl(w.m, row, 64), l = __shfl(w.l, row, 64);
+            if (row >= n) continue;
+            const int h = h0 + row;
+            if (a.splits == 1) {
+                const float fin = finish_row<true>(a, h, m, l);
+#pragma unroll
+                for (int cb = 0; cb < WaveAttn<HD>::CB; ++cb) {
+                    const int d = 16 * cb + li;
+                    if (d < a.vd) store_out<bf16>(a, tok, h, d, w.o[cb][r] * fin);
+                }
+            } else {
+                float* po = a.part_o + (((size_t)item * a.nh + h) * a.splits + split) * a.vd;
+#pragma unroll
+                for (int cb = 0; cb < WaveAttn<HD>::CB; ++cb) {
+                    const int d = 16 * cb + li;
+                    if (d < a.vd) po[d] = m == NEG_INF ? 0.f : w.o[cb][r];
+                }
+                if (li == 0) {
+                    float* pml = a.part_ml + (((size_t)item * a.nh + h) * a.splits + split) * 2;
+                    pml[0] = m == NEG_INF ? NEG_INF : m * LN2;
+                    pml[1] = m == NEG_INF ? 0.f : l;
+                }
+            }
+        }
+        return;
+    }
     const int stride = HD + 2;
     float* mine = wave_out + (size_t)wave * n * stride;
     if (row_ok && g == 0) {
@@ -824,29 +856,40 @@ __global__ __launch_bounds__(MAX_THREADS) void attn_mfma_decode_block_kernel(Att
         }
     }
     __syncthreads();
+    // the block's threads are dealt out to the rows in equal shares: each works out its row's maximum, the waves'
+    // weights and the sum once, then takes every per_row-th column
     const int vd = a.vd;
-    for (int idx = threadIdx.x; idx < n * vd; idx += blockDim.x) {
-        const int row = idx / vd, d = idx - row * vd;
-        float m = NEG_INF;
-        for (int u = 0; u < n_waves; ++u) m = fmaxf(m, wave_out[((size_t)u * n + row) * stride + HD]);
-        float l = 0.f, o = 0.f;
-        for (int u = 0; u < n_waves; ++u) {
+    const int per_row = blockDim.x / n;
+    const int row = threadIdx.x / per_row, sub = threadIdx.x - row * per_row;
+    if (row >= n) return;
+    float m = NEG_INF;
+    for (int u = 0; u < n_waves; ++u) m = fmaxf(m, wave_out[((size_t)u * n + row) * stride + HD]);
+    float f[8], l = 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+        f[u] = 0.f;
+        if (u < n_waves) {
             const float* src = wave_out + ((size_t)u * n + row) * stride;
-            const float f = src[HD] == NEG_INF ? 0.f : __builtin_amdgcn_exp2f(src[HD] - m);
-            l += f * src[HD + 1];
-            o += f * src[d];
+            f[u] = src[HD] == NEG_INF ? 0.f : __builtin_amdgcn_exp2f(src[HD] - m);
+            l += f[u] * src[HD + 1];
         }
-        const int h = h0 + row;
-        if (a.splits == 1) {
-            store_out<bf16>(a, tok, h, d, o * finish_row<true>(a, h, m, l));
-        } else {
-            a.part_o[(((size_t)item * a.nh + h) * a.splits + split) * vd + d] = o;
-            if (d == 0) {
-                float* pml = a.part_ml + (((size_t)item * a.nh + h) * a.splits + split) * 2;
-                pml[0] = m == NEG_INF ? NEG_INF : m * LN2;
-                pml[1] = l;
-            }
-        }
+    }
+    const int h = h0 + row;
+    const bool last = a.splits == 1;
+    const float fin = last ? finish_row<true>(a, h, m, l) : 1.f;
+    float* po = a.part_o + (((size_t)item * a.nh + h) * a.splits + split) * vd;
+    for (int d = sub; d < vd; d += per_row) {
+        float o = 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (u < n_waves) o += f[u] * wave_out[((size_t)u * n + row) * stride + d];
+        if (last) store_out<bf16>(a, tok, h, d, o * fin);
+        else po[d] = o;
+    }
+    if (!last && sub == 0) {
+        float* pml = a.part_ml + (((size_t)item * a.nh + h) * a.splits + split) * 2;
+        pml[0] = m == NEG_INF ? NEG_INF : m * LN2;
+        pml[1] = l;
     }
 }
 
