@@ -404,15 +404,28 @@ FX_API int fx_head_norm_kv_write(void* stream, int dtype, const float* qk, long 
 // up-projection | its rotated part) then scores against it as against the key of one shared head.  The value
 // page [page][1][R][slot] receives c transposed: the heads' outputs are sums of latents, which the values'
 // up-projection is applied to afterwards.
+// With `q_src` (the queries' down-projection of the same tokens, [T, Rq] float32, usually the columns beside `down` in
+// one product's output) a second row of blocks norms that latent too, q_out[t] = q_src[t] / rms * q_w in the pages'
+// type: the two norms that follow the down-projection are one launch.
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void latent_kv_write_kernel(
     const float* __restrict__ down, long ldd, const void* __restrict__ w, int w_dtype, float eps,
     const int* __restrict__ positions, const int* __restrict__ token_seq, const int* __restrict__ block_table, int max_blocks,
     T* __restrict__ k_pages, T* __restrict__ v_pages, int R, int rd, int rot, int bs, const float* __restrict__ inv_freq,
-    float magnitude) {
+    float magnitude, const float* __restrict__ q_src, long ldqs, const void* __restrict__ q_w, float q_eps,
+    T* __restrict__ q_out, long ldq, int Rq) {
     __shared__ float red[4];
     const int t = blockIdx.x, tid = threadIdx.x;
+    if (blockIdx.y == 1) {          // the queries' latent
+        const float* xq = q_src + (size_t)t * ldqs;
+        float sq = 0.f;
+        for (int c = tid; c < Rq; c += 256) sq = fmaf(xq[c], xq[c], sq);
+        sq = block_sum<4>(sq, red);
+        const float qs = 1.0f / sqrtf(sq / (float)Rq + q_eps);
+        for (int c = tid; c < Rq; c += 256) from_float(q_out + (size_t)t * ldq + c, xq[c] * qs * load_as_float(q_w, w_dtype, c));
+        return;
+    }
     const float* x = down + (size_t)t * ldd;
     const int pos = positions[t];
     const int page = block_table[(size_t)token_seq[t] * max_blocks + pos / bs], slot = pos % bs;
@@ -442,20 +455,25 @@ __global__ __launch_bounds__(256) void latent_kv_write_kernel(
 FX_API int fx_latent_kv_write(void* stream, int dtype, const float* down, long ldd, const void* w, int w_dtype, float eps,
                               const int* positions, const int* token_seq, const int* block_table, int max_blocks,
                               void* k_pages, void* v_pages, int T, int R, int rd, int rot, int bs, const float* inv_freq,
-                              float magnitude) {
+                              float magnitude, const float* q_src, long ldqs, const void* q_w, float q_eps, void* q_out,
+                              long ldq, int Rq) {
     FX_REQUIRE(T >= 0 && R > 0 && rd >= 0 && bs > 0 && ldd >= R + rd, "latent_kv_write: bad sizes T=%d R=%d rd=%d", T, R, rd);
     FX_REQUIRE(rot >= 0 && rot <= rd && rot % 2 == 0, "latent_kv_write: %d rotated dimensions of %d", rot, rd);
     FX_REQUIRE(inv_freq || rot == 0, "latent_kv_write: a rotation needs the table of its %d frequencies", rot / 2);
     FX_REQUIRE(w_dtype == FX_F32 || w_dtype == FX_BF16, "latent_kv_write: unknown weight dtype %d", w_dtype);
     FX_REQUIRE(k_pages && v_pages && w, "latent_kv_write: pages and the norm's weight are needed");
+    FX_REQUIRE(!q_src || (q_w && q_out && Rq > 0 && ldqs >= Rq && ldq >= Rq), "latent_kv_write: the queries' latent needs a weight, an output and %d columns", Rq);
     if (T == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
+    const dim3 grid(T, q_src ? 2 : 1);
     if (dtype == FX_F32)
-        latent_kv_write_kernel<float><<<T, 256, 0, s>>>(down, ldd, w, w_dtype, eps, positions, token_seq, block_table, max_blocks,
-                                                        (float*)k_pages, (float*)v_pages, R, rd, rot, bs, inv_freq, magnitude);
+        latent_kv_write_kernel<float><<<grid, 256, 0, s>>>(down, ldd, w, w_dtype, eps, positions, token_seq, block_table, max_blocks,
+                                                           (float*)k_pages, (float*)v_pages, R, rd, rot, bs, inv_freq, magnitude,
+                                                           q_src, ldqs, q_w, q_eps, (float*)q_out, ldq, Rq);
     else if (dtype == FX_BF16)
-        latent_kv_write_kernel<bf16><<<T, 256, 0, s>>>(down, ldd, w, w_dtype, eps, positions, token_seq, block_table, max_blocks,
-                                                       (bf16*)k_pages, (bf16*)v_pages, R, rd, rot, bs, inv_freq, magnitude);
+        latent_kv_write_kernel<bf16><<<grid, 256, 0, s>>>(down, ldd, w, w_dtype, eps, positions, token_seq, block_table, max_blocks,
+                                                          (bf16*)k_pages, (bf16*)v_pages, R, rd, rot, bs, inv_freq, magnitude,
+                                                          q_src, ldqs, q_w, q_eps, (bf16*)q_out, ldq, Rq);
     else
         return fx_fail("latent_kv_write: unknown dtype %d", dtype);
     FX_CHECK_LAUNCH("latent_kv_write");

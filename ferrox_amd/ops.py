@@ -62,7 +62,7 @@ _sigs = {
     ("elementwise", "fx_embed"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float],
     ("elementwise", "fx_latent_kv_write"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_int, c_float, c_void_p, c_void_p,
                                             c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p,
-                                            c_float],
+                                            c_float, c_void_p, c_long, c_void_p, c_float, c_void_p, c_long, c_int],
     ("elementwise", "fx_latent_q_rot"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_int, c_int,
                                          c_int, c_int, c_int, c_void_p, c_float],
     ("elementwise", "fx_span_norm_kv_write"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_int,
@@ -281,12 +281,14 @@ def head_norm_kv_write(qk, q_out, v, q_weight, k_weight, eps, positions, token_s
 
 
 def latent_kv_write(down, weight, eps, positions, token_seq, block_table, k_pages, v_pages, kv_rank: int, rot_dim: int,
-                    rotary_dim: int, block_size: int, inv_freq, magnitude: float = 1.0) -> None:
+                    rotary_dim: int, block_size: int, inv_freq, magnitude: float = 1.0, q_latent=None):
     """What a latent-attention layer keeps per position, from the float32 down-projection `down` [T, kv_rank +
     rot_dim]: the first kv_rank columns through an RMS norm with `weight` (the latent c), the last rot_dim with the
     pairs (2i, 2i+1), i < rotary_dim / 2, turned by pos * inv_freq[i] and stretched by `magnitude`.  The key page
     [pages, 1, block_size, kv_rank + rot_dim] receives (c | rotated part), the value page [pages, 1, kv_rank,
-    block_size] c transposed."""
+    block_size] c transposed.  `q_latent` = (rows, weight, eps): the same launch also norms the queries' latent, float32
+    `rows` [T, q_rank] (any row distance, unit inner stride) with a weight of the keys' norm's type, and returns it
+    [T, q_rank] in the pages' type (None without `q_latent`)."""
     T = down.shape[0]
     R, rd = int(kv_rank), int(rot_dim)
     _f32_rows(down, "latent_kv_write: the down-projection", R + rd)
@@ -300,10 +302,21 @@ def latent_kv_write(down, weight, eps, positions, token_seq, block_table, k_page
         raise KernelError(f"latent_kv_write: {rotary_dim} rotated dimensions need {rotary_dim // 2} float32 frequencies")
     if positions.numel() < T or token_seq.numel() < T:
         raise KernelError("latent_kv_write: the step's index tensors are shorter than its tokens")
+    q_rows = q_w = q_out = None
+    q_eps, Rq = 0.0, 0
+    if q_latent is not None:
+        q_rows, q_w, q_eps = q_latent
+        Rq = q_w.numel()
+        if q_rows.dtype != torch.float32 or q_rows.dim() != 2 or q_rows.stride(1) != 1 or q_rows.shape[0] < T or q_rows.shape[1] < Rq \
+                or q_w.dtype != weight.dtype or not q_w.is_contiguous() or Rq < 1:
+            raise KernelError(f"latent_kv_write: the queries' latent {tuple(q_rows.shape)} with a weight of {Rq} ({q_w.dtype})")
+        q_out = torch.empty((T, Rq), dtype=k_pages.dtype, device=k_pages.device)
     _call("elementwise", "fx_latent_kv_write", _stream(), dtype_code(k_pages.dtype), _p(down), down.stride(0), _p(weight),
           dtype_code(weight.dtype), float(eps), _p(_i32(positions, "positions")), _p(_i32(token_seq, "token_seq")),
           _p(_i32(block_table, "block_table")), block_table.shape[1], _p(k_pages), _p(v_pages), T, R, rd, int(rotary_dim),
-          int(block_size), _p(inv_freq), float(magnitude))
+          int(block_size), _p(inv_freq), float(magnitude), _p(q_rows), q_rows.stride(0) if q_rows is not None else 0, _p(q_w),
+          float(q_eps), _p(q_out), q_out.stride(0) if q_out is not None else 0, int(Rq))
+    return q_out
 
 
 def latent_q_rot(q, q_lat, positions, n_heads: int, dim: int, rot_dim: int, rotary_dim: int, kv_rank: int, inv_freq,

@@ -135,12 +135,18 @@ class LatentAttention(Mixer):
         debug.region("latent down")
         down = matmul(x, self.down, epilogue=ops.EPI_STORE_F32)          # float32: the norms read it
         wq, eps = self.q_norm.rms_params()
-        c_q = ops.rmsnorm(down, wq, eps, ctx.act_dtype, width=self.q_rank)
         if self.own_kv and cache.writes:
+            # one launch: the keys' latent normed, the shared key part rotated, both written; the queries' latent normed
             debug.region("rope + cache write")
             wkv, eps_kv = self.kv_norm.rms_params()
-            ops.latent_kv_write(down[:, self.q_rank:], wkv, eps_kv, ctx.positions, ctx.token_seq, table, k_pages, v_pages,
-                                R, P, self.rot.rotary_dim, cache.block_size, self.inv_freq, self.rot.magnitude)
+            fused = wq.dtype == wkv.dtype and k_pages.dtype == ctx.act_dtype
+            c_q = ops.latent_kv_write(down[:, self.q_rank:], wkv, eps_kv, ctx.positions, ctx.token_seq, table, k_pages, v_pages,
+                                      R, P, self.rot.rotary_dim, cache.block_size, self.inv_freq, self.rot.magnitude,
+                                      q_latent=(down, wq, eps) if fused else None)
+            if not fused:
+                c_q = ops.rmsnorm(down, wq, eps, ctx.act_dtype, width=self.q_rank)
+        else:
+            c_q = ops.rmsnorm(down, wq, eps, ctx.act_dtype, width=self.q_rank)
         debug.region("latent up")
         q = self.up_q(c_q)                                                # [T, H * (D + P)]
         q_lat = torch.empty((T, H * (R + P)), dtype=q.dtype, device=q.device)

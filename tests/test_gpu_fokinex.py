@@ -178,8 +178,19 @@ def test_latent_cache_write_and_query_rotation(dtype):
     kp = torch.zeros(n_pages + 1, 1, bs, R + P, dtype=dt, device="cuda")
     vp = torch.zeros(n_pages + 1, 1, R, bs, dtype=dt, device="cuda")
     inv = ops.rotary_frequencies("cuda", rot, 50.0, tuple(freqs))
-    ops.latent_kv_write(down.cuda()[:, 5:], w.cuda(), 1e-5, pos.cuda(), torch.zeros(T, dtype=torch.int32, device="cuda"),
-                        table.cuda(), kp, vp, R, P, rot, bs, inv, mag)
+    # (the first five columns stand for the queries' latent, which the same launch norms with a weight of its own)
+    wq = (1.0 + 0.2 * torch.randn(5, generator=gen)).to(dt)
+    down_d = down.cuda()
+    assert ops.latent_kv_write(down_d[:, 5:], w.cuda(), 1e-5, pos.cuda(), torch.zeros(T, dtype=torch.int32, device="cuda"),
+                               table.cuda(), kp, vp, R, P, rot, bs, inv, mag) is None
+    kp_alone, vp_alone = kp.clone(), vp.clone()
+    kp.zero_(), vp.zero_()
+    cq = ops.latent_kv_write(down_d[:, 5:], w.cuda(), 1e-5, pos.cuda(), torch.zeros(T, dtype=torch.int32, device="cuda"),
+                             table.cuda(), kp, vp, R, P, rot, bs, inv, mag, q_latent=(down_d, wq.cuda(), 3e-5))
+    assert torch.equal(kp, kp_alone) and torch.equal(vp, vp_alone)
+    assert cq.shape == (T, 5) and cq.dtype == dt
+    want_q = plain.rms_norm(down[:, :5].double(), wq.double(), 3e-5)
+    assert float((cq.double().cpu() - want_q).abs().max()) < (1e-5 if dtype == "float32" else 2e-2)
     c = plain.rms_norm(down[:, 5:5 + R].double(), w.double(), 1e-5)
     kr = plain.rotate_pairs(down[:, 5 + R:].double(), pos.tolist(), freqs, mag)
     tol = 1e-5 if dtype == "float32" else 2e-2
