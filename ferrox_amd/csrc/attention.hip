@@ -442,18 +442,24 @@ __device__ __forceinline__ float quad_sum(float x) {
 }
 
 // A lane's 16 raw scores sc[kb][r] of keys key0 + 4*kb + r, scaled, capped and less the head's penalty for the
-// distance from the row's query at qpos (`shaped_score` with a tanh made of one exponential, whose error, some
-// 1e-7 of the cap, is far below what bfloat16 operands leave of a score): afterwards they are scores in natural
+// distance from the row's query at qpos (`shaped_score` with a tanh made of one exponential and one reciprocal, whose
+// error, some 1e-7 of the cap, is far below what bfloat16 operands leave of a score): afterwards they are scores in natural
 // units, and the softmax step takes them with c = log2(e).
 __device__ __forceinline__ void shape_scores(f32x4_t (&sc)[4], int key0, const AttnArgs& a, float slope, int qpos) {
-    const float inv_cap = a.softcap > 0.f ? 1.f / a.softcap : 0.f;
+    // tanh(x) = 1 - 2 / (1 + e^2x): the exponent in base 2 with the scale folded in, the quotient from the hardware's
+    // reciprocal (1 ulp), cap and -2 cap as the multiply-add's constants
+    const bool capped = a.softcap > 0.f;
+    const float to_exp = capped ? 2.f * a.scale * LOG2E / a.softcap : 0.f;
+    const float cap = a.softcap, cap2 = -2.f * a.softcap;
+    const float d0 = (float)(qpos - key0);
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            float s = sc[kb][r] * a.scale;
-            if (a.softcap > 0.f) s = a.softcap * (1.f - 2.f / (1.f + __expf(2.f * s * inv_cap)));
-            sc[kb][r] = fmaf(-slope, (float)(qpos - (key0 + 4 * kb + r)), s);
+            float s;
+            if (capped) s = fmaf(cap2, __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(sc[kb][r] * to_exp)), cap);
+            else s = sc[kb][r] * a.scale;
+            sc[kb][r] = fmaf(-slope, d0 - (float)(4 * kb + r), s);
         }
 }
 
