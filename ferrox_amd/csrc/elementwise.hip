@@ -483,10 +483,11 @@ FX_API int fx_latent_kv_write(void* stream, int dtype, const float* down, long l
 // The rotated part of the queries of latent attention: q [T, nh * (D + rd)] holds per head D dimensions that are
 // not rotated and rd that are; the rd are turned as the shared key part is (pairs (2i, 2i+1), i < rot / 2, by
 // pos * inv_freq[i], stretched by `magnitude`) and written behind the first R columns of that head's row of
-// q_lat [T, nh * (R + rd)] (the first R columns receive the unrotated part times the keys' up-projection from a
-// matrix product).  One block per token.
+// q_lat [T, nh * (R + rd)] (the first R columns hold the unrotated part taken through the keys' up-projection, from a
+// matrix product).  q_lat may be q itself (D = R: rotation in place; a thread reads the elements it writes, and no
+// other).  One block per token.
 template <typename T>
-__global__ __launch_bounds__(256) void latent_q_rot_kernel(const T* __restrict__ q, long ldq, T* __restrict__ q_lat, long ldl,
+__global__ __launch_bounds__(256) void latent_q_rot_kernel(const T* q, long ldq, T* q_lat, long ldl,
                                                            const int* __restrict__ positions, int nh, int D, int rd, int rot, int R,
                                                            const float* __restrict__ inv_freq, float magnitude) {
     __shared__ float cs[128], sn[128];

@@ -9,10 +9,11 @@ of V, latents of Rq (queries) and R (keys and values):
     score_h(t) = (q_h[:D] . W_uk,h c_t + rot(q_h[D:]) . kr_t) * scale
     y = W_o concat_h( sum_t p_h(t) W_uv,h c_t )                      p: softmax over the window, optionally with a sink
 The cache holds (c | kr) per position and nothing per head.  The kernels never make k_h and v_h: since
-q_h[:D] . W_uk,h c = (W_uk,h^T q_h[:D]) . c, every query head is taken through the transpose of its key
-up-projection, and the attention kernels then see H query heads of R + P dimensions over ONE key head (c | kr) whose
-values are c; the heads' outputs, sums of latents, go through W_uv,h afterwards.  The two per-head products are one
-grouped launch each (a head is a group of rows).  A mixer with `own_kv` False has no W_dkv: its schedule entry reads
+q_h[:D] . W_uk,h c = (W_uk,h^T W_uq,h[:D] c_q) . c, the queries' up-projection is multiplied with the transposes of the
+heads' key up-projections once, when the weights are loaded (in float32, then kept in the weights' type), and one
+product takes c_q to H query heads of [R absorbed | P to be rotated]; the attention kernels then see H query heads of
+R + P dimensions over ONE key head (c | kr) whose values are c; the heads' outputs, sums of latents, go through
+W_uv,h afterwards (one grouped launch in which a head is a group of rows).  A mixer with `own_kv` False has no W_dkv: its schedule entry reads
 the cache of a layer that has one, with W_uk, W_uv, queries, mask and sink of its own.
 """
 from __future__ import annotations
@@ -90,7 +91,7 @@ class LatentAttention(Mixer):
         if self.q_norm.rms_params() is None:
             raise ValueError("latent attention norms its latents with an RMS norm that has a weight")
         self.q_width = self.n_heads * (self.head_dim + self.rot_dim)
-        self.down = self.up_q = self.uk_t = self.uv = self.o_proj = self.sinks = self.inv_freq = None
+        self.down = self.up_q = self.uv = self.o_proj = self.sinks = self.inv_freq = None
 
     def children(self):
         n = self.names
@@ -111,9 +112,12 @@ class LatentAttention(Mixer):
         n, H = self.names, self.n_heads
         # one matrix makes both down-projections: the rows of W_dq, then (a mixer with keys of its own) of W_dkv
         self.down = torch.cat([fetch(n["dq"])] + ([fetch(n["dkv"])] if self.own_kv else []), dim=0).contiguous()
-        self.up_q = Linear(fetch(n["uq"]))
-        # queries go through the transposes of the heads' key up-projections: [H, kv_rank, head_dim]
-        self.uk_t = fetch(n["uk"]).view(H, self.head_dim, self.kv_rank).transpose(1, 2).contiguous()
+        # per head, rows [R: W_uk,h^T W_uq,h[:D] | P: W_uq,h[D:]]: c_q goes straight to what the attention kernels read
+        D, P, R = self.head_dim, self.rot_dim, self.kv_rank
+        uq = fetch(n["uq"]).view(H, D + P, self.q_rank)
+        uk_t = fetch(n["uk"]).view(H, D, R).transpose(1, 2)
+        absorbed = torch.bmm(uk_t.float(), uq[:, :D].float()).to(uq.dtype)                  # [H, R, q_rank]
+        self.up_q = Linear(torch.cat([absorbed, uq[:, D:]], dim=1).reshape(H * (R + P), self.q_rank).contiguous())
         self.uv = fetch(n["uv"]).view(H, self.v_dim, self.kv_rank).contiguous()
         self.o_proj = Linear(fetch(n["o"]))
         if self.has_sink:
@@ -148,13 +152,10 @@ class LatentAttention(Mixer):
         else:
             c_q = ops.rmsnorm(down, wq, eps, ctx.act_dtype, width=self.q_rank)
         debug.region("latent up")
-        q = self.up_q(c_q)                                                # [T, H * (D + P)]
-        q_lat = torch.empty((T, H * (R + P)), dtype=q.dtype, device=q.device)
-        rows, offsets = head_groups(q.device, T, H)
-        # head h of token t: row t*H + h of [T*H, D + P] and of [T*H, R + P]; its first D columns times W_uk,h
-        ops.gemm(q.view(T * H, D + P)[:, :D], self.uk_t, a_rows=rows, c_rows=rows, expert_offsets=offsets, n_rows=T * H,
-                 out=q_lat.view(T * H, R + P)[:, :R])
-        ops.latent_q_rot(q, q_lat, ctx.positions, H, D, P, self.rot.rotary_dim, R, self.inv_freq, self.rot.magnitude)
+        q_lat = self.up_q(c_q)                                            # [T, H * (R + P)]: absorbed parts, parts to rotate
+        q = q_lat
+        if self.rot.rotary_dim:                                           # (in place: a pair is read and written by one thread)
+            ops.latent_q_rot(q_lat, q_lat, ctx.positions, H, R, P, self.rot.rotary_dim, R, self.inv_freq, self.rot.magnitude)
         debug.region("attention")
         out = torch.empty((T, H * R), dtype=q.dtype, device=q.device)
         items = ctx.memo("attention_items 64", lambda: attention_items(ctx, 64))
@@ -168,6 +169,8 @@ class LatentAttention(Mixer):
                                  *common, max_kv_len=items["max_kv"], **extras)
         debug.region("latent values")
         heads = torch.empty((T, H * V), dtype=q.dtype, device=q.device)
+        rows, offsets = head_groups(q.device, T, H)
+        # head h of token t: row t*H + h of [T*H, R] and of [T*H, V]
         ops.gemm(out.view(T * H, R), self.uv, a_rows=rows, c_rows=rows, expert_offsets=offsets, n_rows=T * H,
                  out=heads.view(T * H, V))
         debug.region("o_proj")

@@ -131,9 +131,13 @@ def make_weights(cfg: dict, seed: int) -> dict:
 
 
 # (bfloat16: a layer of this design adds two sublayers' outputs, made from one normed row, to the stream at once, and
-# its latents are few numbers that every head reads; the roundings of seven such layers reach 0.05 of a row's spread
-# at single positions, the same position whatever the cut or the batch.  float32 is the sharp test.)
-LIMIT = {"float32": 3e-5, "bfloat16": 6e-2}
+# its latents are few numbers that every head reads; the roundings of seven such layers reach 0.05 to 0.08 of a row's
+# spread at single positions, the same position whatever the cut or the batch, and which position it is changes with
+# the order of the roundings (random configurations of real layer sizes stay below 0.08 too).  float32 is the sharp
+# test.  EDGE_LIMIT: for models with peaked softmaxes, whose rounding errors are larger, and for one engine run
+# against another.)
+LIMIT = {"float32": 3e-5, "bfloat16": 1e-1}
+EDGE_LIMIT = {"float32": 6e-5, "bfloat16": 1.2e-1}
 
 
 def check_against_plain(cfg, weights, requests, got, dtype, what="", limit=None):
