@@ -1320,8 +1320,9 @@ FX_API int fx_debug_set(const char* key, int value) {
     return 1;
 }
 
-// (value heads narrower than key heads, vd < hd in multiples of 16, run on the kernels in which a wave fetches its own
-// operands: attn_mfma_tile_kernel and attn_mfma_decode_block_kernel)
+// (value heads narrower than key heads, vd < hd in multiples of 16: attn_mfma_tile_kernel and
+// attn_mfma_decode_block_kernel, in which a wave fetches its own operands, and for heads wider than 128
+// attn_mfma_block_kernel<256>, which stages them in LDS; heads beyond HD_MAX go to the kernels for any shape)
 static bool mfma_ok(int dtype, int hd, int bs, const void* q, long ldq, const void* k_pages, const void* v_pages, int vd = 0) {
     return hd <= HD_MAX && (vd == 0 || vd == hd || (vd < hd && vd % 16 == 0)) && dtype == FX_BF16 && hd % 16 == 0 && bs % 16 == 0 && hd % 8 == 0 && ldq % 8 == 0 &&
            (((uintptr_t)q | (uintptr_t)k_pages | (uintptr_t)v_pages) % 16 == 0);
