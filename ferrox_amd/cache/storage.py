@@ -2,7 +2,7 @@
 
 Each schedule entry with a cache of its own gets, for every page tensor its
 mixer names, a slab [num_pages + 1, *page_shape], and for every state tensor a slab
-[n_slots + 1, *state_shape].  An entry that reads another entry's cache sees that
+[n_slots + 1, *state_shape] (a block's own state tensors lie beside its mixer's, as `block.<name>`).  An entry that reads another entry's cache sees that
 entry's page slabs, read-only.  The one page and the one slot past the manager's
 own belong to no request: the stand-in rows that fill a recorded decode step up
 to its fixed number of sequences write there (`pad_page`, `pad_slot`).
@@ -26,7 +26,9 @@ class CacheStorage:
             shapes = mixer.page_shapes(bs)
             key = mixer.cache_group()[0] if shapes else None
             state = {}
-            for name, (shape, sdtype) in mixer.state_shapes().items():
+            block = model.blocks[e.layer]
+            own = {f"block.{name}": v for name, v in block.state_shapes().items()} if hasattr(block, "state_shapes") else {}
+            for name, (shape, sdtype) in {**mixer.state_shapes(), **own}.items():
                 state[name] = torch.zeros((manager.slots.n_slots + 1, *shape), dtype=sdtype or dtype, device=device)
                 self.bytes += state[name].numel() * state[name].element_size()
             if e.cache is not None:

@@ -12,13 +12,14 @@ int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void* out, l
                   const void* v_pages, const int* block_table, int max_blocks, const int* positions, const int* item_seq,
                   const int* item_tok, const int* item_n, int n_items, int nh, int nkv, int hd, int bs, int window, float scale,
                   int tile_q, int vd, int mask_chunk, int keep_first, const float* sinks, const void* gate, long ldg,
-                  float softcap, const float* slopes);
+                  float softcap, const float* slopes, int gate_per_head);
 
 // `vd`: size of a value (and output) head, 0 for hd; part_o is then [n_items, nh, splits, vd].  `mask_chunk` > 0: a query
 // at position p sees the keys t <= p with floor(t / mask_chunk) == floor(p / mask_chunk) (instead of a window).
 // `keep_first` > 0 (with a window): the keys t < keep_first stay visible to every later query.  `sinks` (float32
 // [nh] or null): exp(sinks[h]) joins the denominator of head h's softmax.  `gate` ([tokens, nh * vd], leading
-// dimension ldg, type of `out`; or null): the output is multiplied by sigmoid(gate).  `softcap` > 0: a scaled score s
+// dimension ldg, type of `out`; or null): the output is multiplied by sigmoid(gate); with `gate_per_head` the gate is
+// [tokens, nh], one number for all outputs of a head.  `softcap` > 0: a scaled score s
 // becomes softcap * tanh(s / softcap).  `slopes` (float32 [nh] or null): the score of key t for the query at
 // position p then loses slopes[h] * (p - t).
 // Single queries.  The keys are cut into `splits` chunks of `chunk` positions; the chunks' partial results go through
@@ -27,7 +28,7 @@ int fx_attn_decode(void* stream, int dtype, const void* q, long ldq, void* out, 
                    const void* v_pages, const int* block_table, int max_blocks, const int* positions, const int* item_seq,
                    const int* item_tok, int n_items, int nh, int nkv, int hd, int bs, int window, float scale,
                    float* part_o, float* part_ml, int splits, int chunk, int waves, int vd, int mask_chunk, int keep_first,
-                   const float* sinks, const void* gate, long ldg, float softcap, const float* slopes);
+                   const float* sinks, const void* gate, long ldg, float softcap, const float* slopes, int gate_per_head);
 
 // The same for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops,
 // harnesses that forbid hipMalloc.  It has no counterpart in the reference.  The partial results live in an array

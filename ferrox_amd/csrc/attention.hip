@@ -44,6 +44,7 @@ struct AttnArgs {
     const float* sinks;  // [n_heads] or null: a logit per head that joins the softmax's denominator
     const void* gate;    // [tokens, n_heads * vd] or null (type of out): the output is multiplied by sigmoid(gate)
     long ldg;
+    int gate_per_head;   // 1: the gate is [tokens, n_heads], one number for all of a head's outputs
     float softcap;       // > 0: a scaled score s becomes softcap * tanh(s / softcap)
     const float* slopes; // [n_heads] or null: the score of key t for the query at p then loses slopes[h] * (p - t)
     int bs_shift;        // log2(bs) if bs is a power of two, else -1
@@ -116,7 +117,7 @@ __device__ __forceinline__ float finish_row(const AttnArgs& a, int h, float m, f
 template <typename T>
 __device__ __forceinline__ void store_out(const AttnArgs& a, int tok, int h, int d, float v) {
     if (a.gate) {
-        const float gv = to_float(((const T*)a.gate)[(size_t)tok * a.ldg + (size_t)h * a.vd + d]);
+        const float gv = to_float(((const T*)a.gate)[(size_t)tok * a.ldg + (a.gate_per_head ? (size_t)h : (size_t)h * a.vd + d)]);
         v *= 1.f / (1.f + expf(-gv));
     }
     from_float((T*)a.out + (size_t)tok * a.ldo + (size_t)h * a.vd + d, v);
@@ -1358,7 +1359,7 @@ FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void*
                          const int* positions, const int* item_seq, const int* item_tok, const int* item_n,
                          int n_items, int nh, int nkv, int hd, int bs, int window, float scale, int tile_q,
                          int vd, int mask_chunk, int keep_first, const float* sinks, const void* gate, long ldg,
-                         float softcap, const float* slopes) {
+                         float softcap, const float* slopes, int gate_per_head) {
     if (vd <= 0) vd = hd;
     FX_REQUIRE(softcap >= 0.f && softcap < INFINITY, "attn_tiles: a cap of %g on the scores", (double)softcap);
     if (check_common("attn_tiles", dtype, nh, nkv, hd, bs, window, scale, vd, mask_chunk, keep_first)) return 1;
@@ -1372,6 +1373,7 @@ FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void*
     a.nh = nh; a.nkv = nkv; a.hd = hd; a.bs = bs; a.window = window; a.scale = scale;
     a.vd = vd; a.mask_chunk = mask_chunk;
     a.keep_first = window > 0 ? keep_first : 0; a.sinks = sinks; a.gate = gate; a.ldg = ldg;
+    a.gate_per_head = gate_per_head ? 1 : 0;
     a.softcap = softcap; a.slopes = slopes;
     a.bs_shift = log2_or_minus_one(bs);
     a.n_items = n_items;
@@ -1422,10 +1424,10 @@ static int attn_decode_launch(void* stream, int dtype, const void* q, long ldq, 
                               int nh, int nkv, int hd, int bs, int window, float scale,
                               float* part_o, float* part_ml, int splits, int chunk, int waves, int vd = 0, int mask_chunk = 0,
                               int keep_first = 0, const float* sinks = nullptr, const void* gate = nullptr, long ldg = 0,
-                              float softcap = 0.f, const float* slopes = nullptr) {
+                              float softcap = 0.f, const float* slopes = nullptr, int gate_per_head = 0) {
     if (vd <= 0) vd = hd;
     AttnArgs a = {};
-    a.softcap = softcap; a.slopes = slopes;
+    a.softcap = softcap; a.slopes = slopes; a.gate_per_head = gate_per_head ? 1 : 0;
     a.q = q; a.ldq = ldq; a.out = out; a.ldo = ldo; a.k_pages = k_pages; a.v_pages = v_pages;
     a.block_table = block_table; a.max_blocks = max_blocks; a.positions = positions;
     a.item_seq = item_seq; a.item_tok = item_tok; a.item_n = nullptr;
@@ -1491,14 +1493,15 @@ FX_API int fx_attn_decode(void* stream, int dtype, const void* q, long ldq, void
                           const int* positions, const int* item_seq, const int* item_tok, int n_items,
                           int nh, int nkv, int hd, int bs, int window, float scale,
                           float* part_o, float* part_ml, int splits, int chunk, int waves, int vd, int mask_chunk,
-                          int keep_first, const float* sinks, const void* gate, long ldg, float softcap, const float* slopes) {
+                          int keep_first, const float* sinks, const void* gate, long ldg, float softcap, const float* slopes,
+                          int gate_per_head) {
     if (attn_decode_check(dtype, nh, nkv, hd, bs, window, scale, splits, chunk)) return 1;
     FX_REQUIRE(softcap >= 0.f && softcap < INFINITY, "attn_decode: a cap of %g on the scores", (double)softcap);
     if (check_common("attn_decode", dtype, nh, nkv, hd, bs, window, scale, vd, mask_chunk, keep_first)) return 1;
     if (n_items <= 0) return 0;
     return attn_decode_launch(stream, dtype, q, ldq, out, ldo, k_pages, v_pages, block_table, max_blocks, positions,
                               item_seq, item_tok, n_items, nh, nkv, hd, bs, window, scale, part_o, part_ml, splits,
-                              chunk, waves, vd, mask_chunk, keep_first, sinks, gate, ldg, softcap, slopes);
+                              chunk, waves, vd, mask_chunk, keep_first, sinks, gate, ldg, softcap, slopes, gate_per_head);
 }
 
 // ---------------------------------------------------------------------------

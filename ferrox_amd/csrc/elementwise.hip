@@ -14,29 +14,109 @@ FX_DEFINE_LAST_ERROR()
 // ---------------------------------------------------------------------------
 template <typename W>
 __global__ void embed_kernel(const W* __restrict__ table, const int* __restrict__ ids,
-                             float* __restrict__ h, int H, int V, float scale) {
+                             float* __restrict__ h, int H, int V, float scale,
+                             const W* __restrict__ pos_table, const int* __restrict__ positions, int n_pos) {
     const int t = blockIdx.x;
     int id = ids[t];
-    if (id < 0 || id >= V) {  // the host rejects such ids; never read outside the table
+    const int pos = pos_table ? positions[t] : 0;
+    if (id < 0 || id >= V || pos < 0 || (pos_table && pos >= n_pos)) {  // the host rejects such ids and places; never read outside a table
         for (int c = threadIdx.x; c < H; c += blockDim.x) h[(size_t)t * H + c] = __int_as_float(0x7fc00000);
         return;
     }
     const W* row = table + (size_t)id * H;
+    if (pos_table) {       // a learned vector per position joins the token's row (it is not scaled)
+        const W* prow = pos_table + (size_t)pos * H;
+        for (int c = threadIdx.x; c < H; c += blockDim.x) h[(size_t)t * H + c] = to_float(row[c]) * scale + to_float(prow[c]);
+        return;
+    }
     for (int c = threadIdx.x; c < H; c += blockDim.x) h[(size_t)t * H + c] = to_float(row[c]) * scale;
 }
 
 FX_API int fx_embed(void* stream, int w_dtype, const void* table, const int* ids, float* h,
-                    int T, int H, int V, float scale) {
+                    int T, int H, int V, float scale, const void* pos_table, const int* positions, int n_pos) {
     FX_REQUIRE(T >= 0 && H > 0 && V > 0, "embed: bad sizes T=%d H=%d V=%d", T, H, V);
+    FX_REQUIRE(!pos_table || (positions && n_pos > 0), "embed: a table of positions needs the tokens' positions");
     if (T == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     if (w_dtype == FX_F32)
-        embed_kernel<float><<<T, 256, 0, s>>>((const float*)table, ids, h, H, V, scale);
+        embed_kernel<float><<<T, 256, 0, s>>>((const float*)table, ids, h, H, V, scale, (const float*)pos_table, positions, n_pos);
     else if (w_dtype == FX_BF16)
-        embed_kernel<bf16><<<T, 256, 0, s>>>((const bf16*)table, ids, h, H, V, scale);
+        embed_kernel<bf16><<<T, 256, 0, s>>>((const bf16*)table, ids, h, H, V, scale, (const bf16*)pos_table, positions, n_pos);
     else
         return fx_fail("embed: unknown table dtype %d", w_dtype);
     FX_CHECK_LAUNCH("embed");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Layer norm with weight and bias: y = (x - mean) / sqrt(var + eps) * w + b, var the mean of the squared
+// deviations from the mean (two passes over the row, which the second finds in cache), all in float32.  Input rows are
+// float32 (the residual stream), optionally gathered through `rows`; output is T.  One block per row.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void layernorm_kernel(const float* __restrict__ h, const int* __restrict__ rows,
+                                                        const void* __restrict__ w, const void* __restrict__ b, int w_dtype,
+                                                        T* __restrict__ out, int H, float eps, long ld) {
+    __shared__ float red[4];
+    const int r = blockIdx.x;
+    const float* x = h + (size_t)(rows ? rows[r] : r) * ld;
+    float sum = 0.f;
+    for (int c = threadIdx.x; c < H; c += 256) sum += x[c];
+    const float mean = block_sum<4>(sum, red) / (float)H;
+    __syncthreads();                                   // (`red` is used again)
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < H; c += 256) {
+        const float d = x[c] - mean;
+        ss = fmaf(d, d, ss);
+    }
+    const float rstd = 1.0f / sqrtf(block_sum<4>(ss, red) / (float)H + eps);
+    for (int c = threadIdx.x; c < H; c += 256)
+        from_float(out + (size_t)r * H + c, (x[c] - mean) * rstd * load_as_float(w, w_dtype, c) + (b ? load_as_float(b, w_dtype, c) : 0.f));
+}
+
+FX_API int fx_layernorm(void* stream, int out_dtype, const float* h, const int* rows, const void* w, const void* b,
+                        int w_dtype, void* out, int R, int H, float eps, long ld) {
+    FX_REQUIRE(R >= 0 && H > 0 && w, "layernorm: bad sizes R=%d H=%d", R, H);
+    if (ld == 0) ld = H;
+    FX_REQUIRE(ld >= H, "layernorm: rows %ld apart hold fewer than %d columns", ld, H);
+    FX_REQUIRE(w_dtype == FX_F32 || w_dtype == FX_BF16, "layernorm: unknown weight dtype %d", w_dtype);
+    if (R == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (out_dtype == FX_F32) layernorm_kernel<float><<<R, 256, 0, s>>>(h, rows, w, b, w_dtype, (float*)out, H, eps, ld);
+    else if (out_dtype == FX_BF16) layernorm_kernel<bf16><<<R, 256, 0, s>>>(h, rows, w, b, w_dtype, (bf16*)out, H, eps, ld);
+    else return fx_fail("layernorm: unknown output dtype %d", out_dtype);
+    FX_CHECK_LAUNCH("layernorm");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// h += y * sigmoid(g): a sublayer's float32 output rows pass a learned gate, element by element, as they join the
+// residual stream.  g holds the gate's logits (float32, a product with its bias added).
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void gated_add_kernel(float* __restrict__ h, const float* __restrict__ y,
+                                                        const float* __restrict__ g, long n) {
+    const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i + 3 < n) {
+        const float4 yv = *(const float4*)(y + i), gv = *(const float4*)(g + i);
+        float4 hv = *(const float4*)(h + i);
+        hv.x += yv.x / (1.0f + expf(-gv.x));
+        hv.y += yv.y / (1.0f + expf(-gv.y));
+        hv.z += yv.z / (1.0f + expf(-gv.z));
+        hv.w += yv.w / (1.0f + expf(-gv.w));
+        *(float4*)(h + i) = hv;
+        return;
+    }
+    for (long e = i; e < n; ++e) h[e] += y[e] / (1.0f + expf(-g[e]));
+}
+
+FX_API int fx_gated_add(void* stream, float* h, const float* y, const float* g, long n) {
+    FX_REQUIRE(n >= 0, "gated_add: %ld elements", n);
+    FX_REQUIRE((((uintptr_t)h | (uintptr_t)y | (uintptr_t)g) % 16) == 0, "gated_add: rows must start at multiples of 16 bytes");
+    if (n == 0) return 0;
+    const long blocks = (n + 1023) / 1024;
+    FX_REQUIRE(blocks < (1L << 31), "gated_add: too many elements for one launch");
+    gated_add_kernel<<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>(h, y, g, n);
+    FX_CHECK_LAUNCH("gated_add");
     return 0;
 }
 
@@ -391,6 +471,122 @@ FX_API int fx_head_norm_kv_write(void* stream, int dtype, const float* qk, long 
     else
         return fx_fail("head_norm_kv_write: unknown dtype %d", dtype);
     FX_CHECK_LAUNCH("head_norm_kv_write");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// For attention that rotates nothing, warms its queries with the position and keeps values of unit size.  From the
+// float32 product qkv [T, nh hd | nkv hd | nkv vd | n_gate] of a token at position p:
+//   q_out[:, :nh hd]  = q * (1 + coef ln(floor((p + 1) / every) + 1))          the query's temperature (coef 0: none)
+//   q_out[:, nh hd:]  = the n_gate gate columns, as they are (the attention kernels read them beside the queries)
+//   key page          <- k
+//   value page        <- v / sqrt(mean(v^2) + eps) per head (unit_values), else v; transposed
+// q_out and the pages have type T; temperature and norm are float32 arithmetic.  The first blocks take (token, unit)
+// pairs a wave each, a unit being a head of q, a head of k or the gate columns; the blocks after them take (eight
+// consecutive tokens, kv head): they norm the eight value heads into LDS and write them as `write_values` does.
+// ---------------------------------------------------------------------------
+#define UNIT_VD_MAX 256
+template <typename T>
+__global__ __launch_bounds__(256) void temp_unit_kv_write_kernel(
+    const float* __restrict__ qkv, long ld, T* __restrict__ q_out, long ldq, const int* __restrict__ positions,
+    const int* __restrict__ token_seq, const int* __restrict__ block_table, int max_blocks, T* __restrict__ k_pages,
+    T* __restrict__ v_pages, int n_tokens, int nh, int nkv, int hd, int vd, int bs, int n_gate, float coef, int every,
+    int unit_values, float eps, int head_blocks) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if ((int)blockIdx.x < head_blocks) {
+        const int units = nh + (k_pages ? nkv : 0) + (n_gate ? 1 : 0);
+        const int r = blockIdx.x * 4 + wave;
+        if (r >= n_tokens * units) return;
+        const int t = r / units, u = r - t * units;
+        const float* row = qkv + (size_t)t * ld;
+        if (u < nh) {
+            const int pos = positions[t];
+            const float temp = coef != 0.f ? 1.0f + coef * logf((float)((pos + 1) / every) + 1.0f) : 1.0f;
+            for (int c = lane; c < hd; c += 64) from_float(q_out + (size_t)t * ldq + (size_t)u * hd + c, row[(size_t)u * hd + c] * temp);
+        } else if (k_pages && u < nh + nkv) {
+            const int kh = u - nh, pos = positions[t];
+            const int page = block_table[(size_t)token_seq[t] * max_blocks + pos / bs];
+            T* dst = k_pages + (((size_t)page * nkv + kh) * bs + pos % bs) * hd;
+            for (int c = lane; c < hd; c += 64) from_float(dst + c, row[(size_t)(nh + kh) * hd + c]);
+        } else {
+            const float* g = row + (size_t)(nh + nkv) * hd + (size_t)nkv * vd;
+            for (int c = lane; c < n_gate; c += 64) from_float(q_out + (size_t)t * ldq + (size_t)nh * hd + c, g[c]);
+        }
+        return;
+    }
+    if (!v_pages) return;
+    __shared__ T vs[8][UNIT_VD_MAX];
+    const int b = blockIdx.x - head_blocks;
+    const int kh = b % nkv, t0 = (b / nkv) * 8;
+    const int n = min(8, n_tokens - t0);
+    for (int i = wave; i < n; i += 4) {
+        const float* v = qkv + (size_t)(t0 + i) * ld + (size_t)(nh + nkv) * hd + (size_t)kh * vd;
+        float xv[UNIT_VD_MAX / 64];
+        float ss = 0.f;
+#pragma unroll
+        for (int e = 0; e < UNIT_VD_MAX / 64; ++e) {
+            const int c = lane + e * 64;
+            xv[e] = c < vd ? v[c] : 0.f;
+            ss = fmaf(xv[e], xv[e], ss);
+        }
+        const float scale = unit_values ? 1.0f / sqrtf(wave_sum(ss) / (float)vd + eps) : 1.0f;
+#pragma unroll
+        for (int e = 0; e < UNIT_VD_MAX / 64; ++e) {
+            const int c = lane + e * 64;
+            if (c < vd) from_float(&vs[i][c], xv[e] * scale);
+        }
+    }
+    __syncthreads();
+    const int pos0 = positions[t0], seq0 = token_seq[t0];
+    bool together = sizeof(T) == 2 && n == 8 && (bs & 7) == 0 && (pos0 & 7) == 0;
+    for (int i = 1; together && i < 8; ++i) together = positions[t0 + i] == pos0 + i && token_seq[t0 + i] == seq0;
+    if (together) {      // eight tokens that follow each other in one page: one 16-byte store per value channel
+        const int page = block_table[(size_t)seq0 * max_blocks + pos0 / bs];
+        T* dst = v_pages + ((size_t)page * nkv + kh) * vd * bs + pos0 % bs;
+        for (int d = tid; d < vd; d += 256) {
+            uint16_t e[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) e[i] = *(const uint16_t*)&vs[i][d];
+            uint4 o;
+            o.x = e[0] | ((uint32_t)e[1] << 16);
+            o.y = e[2] | ((uint32_t)e[3] << 16);
+            o.z = e[4] | ((uint32_t)e[5] << 16);
+            o.w = e[6] | ((uint32_t)e[7] << 16);
+            *(uint4*)(dst + (size_t)d * bs) = o;
+        }
+        return;
+    }
+    for (int idx = tid; idx < n * vd; idx += 256) {
+        const int i = idx / vd, d = idx - i * vd;
+        const int t = t0 + i, pos = positions[t];
+        const int page = block_table[(size_t)token_seq[t] * max_blocks + pos / bs];
+        v_pages[(((size_t)page * nkv + kh) * vd + d) * bs + pos % bs] = vs[i][d];
+    }
+}
+
+FX_API int fx_temp_unit_kv_write(void* stream, int dtype, const float* qkv, long ld, void* q_out, long ldq, const int* positions,
+                                 const int* token_seq, const int* block_table, int max_blocks, void* k_pages, void* v_pages,
+                                 int T, int nh, int nkv, int hd, int vd, int bs, int n_gate, float coef, int every,
+                                 int unit_values, float eps) {
+    FX_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && bs > 0 && n_gate >= 0, "temp_unit_kv_write: bad sizes");
+    FX_REQUIRE(hd > 0 && vd > 0 && vd <= UNIT_VD_MAX, "temp_unit_kv_write: head sizes %d and %d (values up to %d)", hd, vd, UNIT_VD_MAX);
+    FX_REQUIRE(every >= 1, "temp_unit_kv_write: a temperature step every %d positions", every);
+    FX_REQUIRE((k_pages == nullptr) == (v_pages == nullptr), "temp_unit_kv_write: key and value pages must come together");
+    FX_REQUIRE(ld >= (long)(nh + nkv) * hd + (long)nkv * vd + n_gate && ldq >= (long)nh * hd + n_gate, "temp_unit_kv_write: rows too short");
+    if (T == 0) return 0;
+    const long units = nh + (k_pages ? nkv : 0) + (n_gate ? 1 : 0);
+    const long head_blocks = (T * units + 3) / 4, n_blocks = head_blocks + (v_pages ? (long)((T + 7) / 8) * nkv : 0);
+    FX_REQUIRE(n_blocks < (1L << 31), "temp_unit_kv_write: too many tokens and heads for one launch");
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == FX_F32)
+        temp_unit_kv_write_kernel<float><<<(unsigned)n_blocks, 256, 0, s>>>(qkv, ld, (float*)q_out, ldq, positions, token_seq, block_table,
+            max_blocks, (float*)k_pages, (float*)v_pages, T, nh, nkv, hd, vd, bs, n_gate, coef, every, unit_values, eps, (int)head_blocks);
+    else if (dtype == FX_BF16)
+        temp_unit_kv_write_kernel<bf16><<<(unsigned)n_blocks, 256, 0, s>>>(qkv, ld, (bf16*)q_out, ldq, positions, token_seq, block_table,
+            max_blocks, (bf16*)k_pages, (bf16*)v_pages, T, nh, nkv, hd, vd, bs, n_gate, coef, every, unit_values, eps, (int)head_blocks);
+    else
+        return fx_fail("temp_unit_kv_write: unknown dtype %d", dtype);
+    FX_CHECK_LAUNCH("temp_unit_kv_write");
     return 0;
 }
 

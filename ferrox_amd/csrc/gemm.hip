@@ -64,6 +64,9 @@ struct GemmArgs {
     const float* rope_freq_factors;   // rot/2 floats or null: the angle of pair i is divided by rope_freq_factors[i]
     int stream_w;  // tiled kernel: the weights are read about once (one row tile a weight matrix): load them non-temporal
     int act;     // EPI_GATED: which activation the gate goes through (ACT_*)
+    float act_limit, act_alpha;   // ACT_SWIGLU_CLAMP: the bound on gate and up, and the sigmoid's slope
+    const float* pre_scale;       // EPI_GATED: [.] or null: gate and up of logical row m are multiplied by
+    const int* pre_scale_rows;    //   pre_scale[pre_scale_rows ? pre_scale_rows[m] : m] before the activation (a row of A scaled)
     int store_act;   // EPI_STORE: what the product goes through before it is stored (SACT_*), 0 for nothing
     int vec_ok;  // 16-byte loads are legal for A and W
     int n_col_tiles, n_row_tiles;  // tiled kernels: the grid they decode block ids with
@@ -177,11 +180,16 @@ __device__ __forceinline__ bool locate_pairs(const GemmArgs& g, int tile, int& e
 //   ACT_GELU_TANH  0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3)))
 //   ACT_GELU       0.5 x (1 + erf(x / sqrt(2)))
 //   ACT_RELU       max(x, 0)
-enum { ACT_SILU = 0, ACT_GELU_TANH = 1, ACT_GELU = 2, ACT_RELU = 3, ACT_COUNT = 4 };
+//   ACT_SWIGLU_CLAMP  g = min(gate, limit), u = clamp(up, -limit, limit): g sigmoid(alpha g) (u + 1)
+enum { ACT_SILU = 0, ACT_GELU_TANH = 1, ACT_GELU = 2, ACT_RELU = 3, ACT_SWIGLU_CLAMP = 4, ACT_COUNT = 5 };
 __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }
 template <int ACT>
-__device__ __forceinline__ float gated_c(float gate, float up) {
+__device__ __forceinline__ float gated_c(float gate, float up, float limit, float alpha) {
     float a;
+    if constexpr (ACT == ACT_SWIGLU_CLAMP) {
+        const float gc = fminf(gate, limit), uc = fminf(fmaxf(up, -limit), limit);
+        return gc / (1.0f + expf(-alpha * gc)) * (uc + 1.0f);
+    }
     if constexpr (ACT == ACT_GELU_TANH) a = 0.5f * gate * (1.0f + tanhf(0.7978845608028654f * (gate + 0.044715f * gate * gate * gate)));
     else if constexpr (ACT == ACT_GELU) a = 0.5f * gate * (1.0f + erff(gate * 0.7071067811865476f));
     else if constexpr (ACT == ACT_RELU) a = fmaxf(gate, 0.0f);
@@ -202,6 +210,8 @@ __device__ __forceinline__ float stored_f(int act, float x) {
     if (act == SACT_SILU) return silu_f(x);
     return 0.5f * x * (1.0f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
 }
+// what gate and up of logical row m are multiplied by before the activation (1 without a pre-scale)
+#define FX_PRE_SCALE(g, ml) ((g).pre_scale ? (g).pre_scale[(g).pre_scale_rows ? (g).pre_scale_rows[ml] : (ml)] : 1.0f)
 // f(the activation as a compile-time constant): an epilogue calls this once around its loops, so that the choice is
 // one jump per block and not work inside the loops (left inside, the compiler works out every activation for every
 // element and picks one: the tiled products of a prompt were 4-10 % slower for it)
@@ -211,6 +221,7 @@ __device__ __forceinline__ void with_activation(int act, F&& f) {
         case ACT_GELU_TANH: f(std::integral_constant<int, ACT_GELU_TANH>{}); break;
         case ACT_GELU: f(std::integral_constant<int, ACT_GELU>{}); break;
         case ACT_RELU: f(std::integral_constant<int, ACT_RELU>{}); break;
+        case ACT_SWIGLU_CLAMP: f(std::integral_constant<int, ACT_SWIGLU_CLAMP>{}); break;
         default: f(std::integral_constant<int, ACT_SILU>{}); break;
     }
 }
@@ -361,11 +372,12 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmArgs g) {
                     const int ml = r0 + wm * WM + i * 16 + (lane >> 4) * 4 + r;
                     if (ml >= r_end) continue;
                     const int m = g.c_rows ? g.c_rows[ml] : ml;
+                    const float ps = FX_PRE_SCALE(g, ml);
 #pragma unroll
                     for (int j = 0; j < NT; j += 2) {
                         const int n = n0 + wn * (WN / 2) + (j / 2) * 16 + (lane & 15);
                         if (n < g.N)
-                            from_float((bf16*)g.C + (size_t)m * g.ldc + n, gated_c<decltype(ac)::value>(acc[i][j][r], acc[i][j + 1][r]));
+                            from_float((bf16*)g.C + (size_t)m * g.ldc + n, gated_c<decltype(ac)::value>(acc[i][j][r] * ps, acc[i][j + 1][r] * ps, g.act_limit, g.act_alpha));
                     }
                 }
         });
@@ -388,7 +400,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmArgs g) {
                     if (EPI == EPI_STORE) {
                         from_float((bf16*)g.C + (size_t)m * g.ldc + n, stored_f(g.store_act, v));
                     } else if (EPI == EPI_STORE_F32) {
-                        ((float*)g.C)[(size_t)m * g.ldc + n] = v;
+                        ((float*)g.C)[(size_t)m * g.ldc + n] = stored_f(g.store_act, v);
                     } else {
                         if (g.row_scale) v *= g.row_scale[ml];
                         ((float*)g.C)[(size_t)m * g.ldc + n] += v;
@@ -615,11 +627,12 @@ __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(GemmArgs g) {
                     const int ml = r0 + (2 * i + wm) * 16 + (lane >> 4) * 4 + r;
                     if (ml >= r_end || ml >= r0 + TM) continue;
                     const int m = m_of[i][r];
+                    const float ps = FX_PRE_SCALE(g, ml);
 #pragma unroll
                     for (int j = 0; j < NT; j += 2) {
                         const int n = n0 + wn * (WN / 2) + (j / 2) * 16 + (lane & 15);
                         if (n < g.N)
-                            from_float((bf16*)g.C + (size_t)m * g.ldc + n, gated_c<decltype(ac)::value>(acc[i][j][r], acc[i][j + 1][r]));
+                            from_float((bf16*)g.C + (size_t)m * g.ldc + n, gated_c<decltype(ac)::value>(acc[i][j][r] * ps, acc[i][j + 1][r] * ps, g.act_limit, g.act_alpha));
                     }
                 }
         });
@@ -652,7 +665,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(GemmArgs g) {
                     if (EPI == EPI_STORE) {
                         from_float((bf16*)g.C + (size_t)m * g.ldc + n, stored_f(g.store_act, v));
                     } else if (EPI == EPI_STORE_F32) {
-                        ((float*)g.C)[(size_t)m * g.ldc + n] = v;
+                        ((float*)g.C)[(size_t)m * g.ldc + n] = stored_f(g.store_act, v);
                     } else {
                         if (g.row_scale) {
                             v *= scale_of[i][r];
@@ -1090,14 +1103,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
             float o = v[r] * rstd;
             asm volatile("" : "+v"(o));          // the product is rounded before the bias is added (no fused multiply-add)
             if (DUAL) {
-                with_activation(g.act, [&](auto ac) { from_float((bf16*)g.C + (size_t)m * g.ldc + n, gated_c<decltype(ac)::value>(o, v2[r])); });
+                const float ps = FX_PRE_SCALE(g, ml);
+                with_activation(g.act, [&](auto ac) { from_float((bf16*)g.C + (size_t)m * g.ldc + n, gated_c<decltype(ac)::value>(o * ps, v2[r] * ps, g.act_limit, g.act_alpha)); });
                 continue;
             }
             if (g.bias) o += bias_v[r];
             if (EPI == EPI_STORE) {
                 from_float((bf16*)g.C + (size_t)m * g.ldc + n, stored_f(g.store_act, o));
             } else if (EPI == EPI_STORE_F32) {
-                ((float*)g.C)[(size_t)m * g.ldc + n] = o;
+                ((float*)g.C)[(size_t)m * g.ldc + n] = stored_f(g.store_act, o);
             } else {
                 if (g.row_scale) {
                     o *= row_scale;
@@ -1186,7 +1200,8 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs g) {
             float v = acc[i][j];
             float* out = (float*)g.C + (size_t)m * g.ldc + n;
             if (DUAL) {
-                with_activation(g.act, [&](auto ac) { *out = gated_c<decltype(ac)::value>(v, acc2[i][j]); });
+                const float ps = FX_PRE_SCALE(g, ml);
+                with_activation(g.act, [&](auto ac) { *out = gated_c<decltype(ac)::value>(v * ps, acc2[i][j] * ps, g.act_limit, g.act_alpha); });
             } else {
                 if (g.bias) v += load_as_float(g.bias, g.bias_dtype, n);
                 if (EPI == EPI_RESID) {
@@ -1379,9 +1394,12 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
                    const float* row_scale, const int* a_rows, const int* c_rows, const int* expert_offsets,
                    int E, int M, int N, int K, const void* norm_w, int norm_dtype, float norm_eps,
                    const int* pair_ids, int pair_div, int n_always, int always_rows, int always_from_a, long kb_rows,
-                   const float* row_ss, int row_ss_n, int act, int store_act) {
-    FX_REQUIRE(store_act >= 0 && store_act < SACT_COUNT && (store_act == 0 || (epi == EPI_STORE && !bias)),
+                   const float* row_ss, int row_ss_n, int act, int store_act, float act_limit, float act_alpha,
+                   const float* pre_scale, const int* pre_scale_rows) {
+    FX_REQUIRE(store_act >= 0 && store_act < SACT_COUNT && (store_act == 0 || ((epi == EPI_STORE || epi == EPI_STORE_F32) && !bias)),
                "gemm: a stored activation (%d) goes with the plain stored product without bias", store_act);
+    FX_REQUIRE(!pre_scale || epi == EPI_GATED, "gemm: a scale in front of the activation goes with the gate/up epilogue");
+    FX_REQUIRE(act != ACT_SWIGLU_CLAMP || act_limit > 0.f, "gemm: the clamped gate needs a positive limit, got %g", (double)act_limit);
     FX_REQUIRE(dtype == FX_F32 || dtype == FX_BF16, "gemm: unknown dtype %d", dtype);
     FX_REQUIRE(epi >= EPI_STORE && epi <= EPI_GATED, "gemm: unknown epilogue %d", epi);
     FX_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
@@ -1411,6 +1429,7 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
     g.bias = bias; g.bias_dtype = bias_dtype; g.C = C; g.ldc = ldc; g.row_scale = row_scale;
     g.a_rows = a_rows; g.c_rows = c_rows; g.expert_offsets = expert_offsets; g.E = E; g.M = M; g.N = N; g.K = K;
     g.pair_ids = pair_ids; g.pair_div = pair_div; g.act = act; g.store_act = store_act;
+    g.act_limit = act_limit; g.act_alpha = act_alpha; g.pre_scale = pre_scale; g.pre_scale_rows = pre_scale_rows;
     g.kb_stride = kb_rows * 64;
     FX_REQUIRE(kb_rows >= 0 && (kb_rows == 0 || (dtype == FX_BF16 && K % 64 == 0 && ((uintptr_t)W % 16) == 0 && lda % 8 == 0 &&
                                                  ((uintptr_t)A % 16) == 0 && (up_offset % K) == 0)),

@@ -39,7 +39,7 @@ class Model:
                 raise ValueError(f"layer {ls.prefix!r}: block '{ls.block}' needs parts {sorted(missing)}"
                                  + (f" and has no place for {sorted(unknown)}" if unknown else ""))
             parts = {slot: reg.build(ls.parts[slot]) for slot, reg in cls.slots.items() if slot in ls.parts}
-            self.blocks.append(cls(parts, {slot: ls.parts[slot].prefix for slot in parts}))
+            self.blocks.append(cls(parts, {slot: ls.parts[slot].prefix for slot in parts}, **ls.args))
         self.final_norm = NORMS.build(spec.final_norm)
         self.head = HEADS.build(spec.head)
         self.schedule = list(spec.schedule)
@@ -126,7 +126,9 @@ class Model:
     # ---- forward ---------------------------------------------------------
     def forward(self, ctx: StepContext, caches: list):
         debug.region("embed")
-        h = self.embedding.forward(ctx.token_ids)
+        # (an embedding that adds something per position says so and gets the tokens' positions)
+        h = self.embedding.forward(ctx.token_ids, positions=ctx.positions) if getattr(self.embedding, "uses_positions", False) \
+            else self.embedding.forward(ctx.token_ids)
         # blocks that chain their norms: the block before may already have applied this block's first norm
         # to the rows it finished (in the kernel that finished them)
         normed = None

@@ -89,6 +89,9 @@ def _register_builtin():
     from ..config.fokinex import FokinexConfig
     from .fokinex import build_spec as fokinex_spec
     register_architecture(Architecture(FokinexConfig.architecture, FokinexConfig.model_type, FokinexConfig, fokinex_spec))
+    from ..config.panarax import PanaraxConfig
+    from .panarax import build_spec as panarax_spec
+    register_architecture(Architecture(PanaraxConfig.architecture, PanaraxConfig.model_type, PanaraxConfig, panarax_spec))
 
 
 _register_builtin()

@@ -18,7 +18,7 @@ from .csrc.build import load_library
 FX_F32, FX_BF16 = 0, 1
 EPI_STORE, EPI_STORE_F32, EPI_RESID, EPI_GATED = 0, 1, 2, 3
 # what the gate of a gated product goes through (EPI_GATED stores activation(gate) * up); ACT_* in csrc/gemm.hip
-ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "gelu": 2, "relu": 3}
+ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "gelu": 2, "relu": 3, "swiglu_clamped": 4}
 # what a stored product (EPI_STORE) may go through on its way out, the activation of a feed-forward without a
 # gate; SACT_* in csrc/gemm.hip
 STORED_ACTIVATIONS = {None: 0, "relu2": 1, "relu": 2, "silu": 3, "gelu_tanh": 4}
@@ -59,7 +59,12 @@ def _stream():
 
 
 _sigs = {
-    ("elementwise", "fx_embed"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float],
+    ("elementwise", "fx_embed"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_int],
+    ("elementwise", "fx_layernorm"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_long],
+    ("elementwise", "fx_gated_add"): [c_void_p, c_void_p, c_void_p, c_void_p, c_long],
+    ("elementwise", "fx_temp_unit_kv_write"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p,
+                                               c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                               c_float, c_int, c_int, c_float],
     ("elementwise", "fx_latent_kv_write"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_int, c_float, c_void_p, c_void_p,
                                             c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p,
                                             c_float, c_void_p, c_long, c_void_p, c_float, c_void_p, c_long, c_int],
@@ -75,8 +80,17 @@ _sigs = {
     ("elementwise", "fx_rmsnorm_add"): [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float],
     ("elementwise", "fx_moe_combine_identity"): [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                                  c_int, c_int, c_int, c_int, c_void_p, c_int, c_float],
-    ("recurrent", "fx_short_conv"): [c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_int, c_void_p,
-                                     c_void_p, c_void_p, c_void_p, c_int, c_int, c_int],
+    ("recurrent", "fx_short_conv"): [c_void_p, c_void_p, c_int, c_long, c_void_p, c_int, c_long, c_void_p, c_int, c_int, c_void_p,
+                                     c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_int],
+    ("recurrent", "fx_gated_outer"): [c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_void_p,
+                                      c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                      c_float],
+    ("recurrent", "fx_exp_gate_scan"): [c_void_p, c_void_p, c_long, c_void_p, c_long, c_float, c_void_p, c_void_p, c_void_p,
+                                        c_void_p, c_void_p, c_void_p, c_int, c_int],
+    ("recurrent", "fx_rglru_gates"): [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_float,
+                                      c_void_p, c_void_p, c_int, c_int, c_int],
+    ("recurrent", "fx_rglru_scan"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p,
+                                     c_void_p, c_int, c_int, c_int],
     ("recurrent", "fx_delta_prepare"): [c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_long, c_void_p, c_long,
                                         c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                         c_int, c_int, c_int, c_int, c_int],
@@ -84,8 +98,8 @@ _sigs = {
                                         c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int],
     ("recurrent", "fx_small_rows_pair"): [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_int,
                                           c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_int, c_int],
-    ("recurrent", "fx_gated_head_norm"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_void_p,
-                                          c_long, c_int, c_int, c_int, c_float, c_int],
+    ("recurrent", "fx_gated_head_norm"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_int, c_void_p,
+                                          c_long, c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p],
     ("elementwise", "fx_head_norm_kv_write"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int,
                                                c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p, c_int,
                                                c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int],
@@ -97,20 +111,21 @@ _sigs = {
     ("elementwise", "fx_feed_tokens"): [c_void_p, c_void_p, c_void_p, c_void_p, c_int],
     ("gemm", "fx_gemm"): [c_void_p, c_int, c_int, c_void_p, c_long, c_void_p, c_long, c_long, c_void_p, c_int,
                           c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                          c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_int, c_long, c_void_p, c_int, c_int, c_int],
+                          c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_int, c_long, c_void_p, c_int, c_int, c_int,
+                          c_float, c_float, c_void_p, c_void_p],
     ("gemm", "fx_qkv_rope"): [c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_void_p, c_long, c_int, c_int,
                               c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p],
     ("attention", "fx_attn_tiles"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p,
                                      c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int,
-                                     c_int, c_void_p, c_void_p, c_long, c_float, c_void_p],
+                                     c_int, c_void_p, c_void_p, c_long, c_float, c_void_p, c_int],
     ("attention", "fx_attn_tile_queries"): [c_int, c_int, c_int],
     ("attention", "fx_attn_decode"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p,
                                       c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                                       c_int, c_int, c_int, c_int, c_int, c_float,
                                       c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                                      c_int, c_void_p, c_void_p, c_long, c_float, c_void_p],
+                                      c_int, c_void_p, c_void_p, c_long, c_float, c_void_p, c_int],
     ("moe", "fx_router_select"): [c_void_p, c_void_p, c_long, c_long, c_int, c_int, c_int, c_int, c_float, c_float, c_int,
                                   c_void_p, c_void_p, c_void_p, c_void_p],
     ("moe", "fx_router_select_align"): [c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_float, c_float, c_int,
@@ -149,15 +164,75 @@ def _i32(t, what):
 
 
 # ---------------------------------------------------------------------------
-def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | None = None, scale: float = 1.0) -> torch.Tensor:
-    """h[t] = table[ids[t]] * scale as float32."""
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | None = None, scale: float = 1.0,
+          position_table: torch.Tensor | None = None, positions: torch.Tensor | None = None) -> torch.Tensor:
+    """h[t] = table[ids[t]] * scale (+ position_table[positions[t]], a learned vector per position) as float32."""
     V, H = table.shape
     T = ids.numel()
     if out is None:
         out = torch.empty((T, H), dtype=torch.float32, device=table.device)
+    n_pos = 0
+    if position_table is not None:
+        if positions is None or positions.numel() < T or position_table.dtype != table.dtype or position_table.dim() != 2 \
+                or position_table.shape[1] != H or not position_table.is_contiguous():
+            raise KernelError(f"embed: a table of positions {tuple(position_table.shape)} ({position_table.dtype}) beside an "
+                              f"embedding table {tuple(table.shape)} ({table.dtype}) needs the tokens' positions")
+        n_pos = position_table.shape[0]
     _call("elementwise", "fx_embed", _stream(), dtype_code(table.dtype), _p(table), _p(_i32(ids, "ids")), _p(out), T, H, V,
-          float(scale))
+          float(scale), _p(position_table), _p(_i32(positions, "positions")) if position_table is not None else None, n_pos)
     return out
+
+
+def layernorm(h: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, eps: float, out_dtype: torch.dtype,
+              rows: torch.Tensor | None = None) -> torch.Tensor:
+    """Rows of float32 `h` (all, or those in `rows`) through (x - mean) / sqrt(var + eps) * weight + bias, var the
+    mean of the squared deviations, into `out_dtype`."""
+    if h.dtype != torch.float32 or h.dim() != 2 or not h.is_contiguous():
+        raise KernelError("layernorm reads contiguous float32 rows")
+    H = h.shape[1]
+    if weight.numel() != H or not weight.is_contiguous() or (bias is not None and (bias.numel() != H or bias.dtype != weight.dtype
+                                                                                     or not bias.is_contiguous())):
+        raise KernelError(f"layernorm: weight and bias must hold {H} elements of one type")
+    R = h.shape[0] if rows is None else rows.numel()
+    out = torch.empty((R, H), dtype=out_dtype, device=h.device)
+    _call("elementwise", "fx_layernorm", _stream(), dtype_code(out_dtype), _p(h), _p(_i32(rows, "rows")), _p(weight), _p(bias),
+          dtype_code(weight.dtype), _p(out), R, H, float(eps), h.stride(0))
+    return out
+
+
+def gated_add(h: torch.Tensor, y: torch.Tensor, gate_logits: torch.Tensor) -> None:
+    """h += y * sigmoid(gate_logits), element by element (contiguous float32 tensors of one shape)."""
+    for t in (h, y, gate_logits):
+        if t.dtype != torch.float32 or not t.is_contiguous() or t.shape != h.shape:
+            raise KernelError("gated_add wants contiguous float32 tensors of one shape")
+    _call("elementwise", "fx_gated_add", _stream(), _p(h), _p(y), _p(gate_logits), h.numel())
+
+
+def temp_unit_kv_write(qkv, q_out, positions, token_seq, block_table, k_pages, v_pages, n_heads: int, n_kv_heads: int,
+                       head_dim: int, v_dim: int, block_size: int, n_gate: int = 0, temperature: tuple | None = None,
+                       unit_values: bool = False, eps: float = 0.0) -> None:
+    """For attention that rotates nothing: from the float32 product qkv [T, nh*hd | nkv*hd | nkv*vd | n_gate], q times the
+    temperature of its position, 1 + coef ln(floor((p + 1) / every) + 1) with `temperature` = (coef, every), into
+    q_out[:, :nh*hd]; the gate columns into q_out[:, nh*hd:]; k into its page; v, each head divided by its root mean
+    square over v_dim (`unit_values`, eps inside the root), into its transposed page.  Pages None: nothing is cached."""
+    T = qkv.shape[0]
+    nh, nkv, hd, vd = int(n_heads), int(n_kv_heads), int(head_dim), int(v_dim)
+    cols = (nh + nkv) * hd + nkv * vd + int(n_gate)
+    _f32_rows(qkv, "temp_unit_kv_write: qkv", cols)
+    if q_out.dim() != 2 or q_out.stride(1) != 1 or q_out.shape[0] < T or q_out.shape[1] < nh * hd + n_gate:
+        raise KernelError(f"temp_unit_kv_write: q_out {tuple(q_out.shape)} for {T} rows of {nh * hd + n_gate}")
+    if (k_pages is None) != (v_pages is None):
+        raise KernelError("temp_unit_kv_write: key and value pages come together")
+    if k_pages is not None and (tuple(k_pages.shape[1:]) != (nkv, block_size, hd) or tuple(v_pages.shape[1:]) != (nkv, vd, block_size)
+                                or k_pages.dtype != q_out.dtype or v_pages.dtype != q_out.dtype):
+        raise KernelError(f"temp_unit_kv_write: pages {tuple(k_pages.shape)}, {tuple(v_pages.shape)} for {nkv} heads of {hd} / {vd}")
+    coef, every = (float(temperature[0]), int(temperature[1])) if temperature else (0.0, 1)
+    if positions.numel() < T or token_seq.numel() < T:
+        raise KernelError("temp_unit_kv_write: the step's index tensors are shorter than its tokens")
+    _call("elementwise", "fx_temp_unit_kv_write", _stream(), dtype_code(q_out.dtype), _p(qkv), qkv.stride(0), _p(q_out),
+          q_out.stride(0), _p(_i32(positions, "positions")), _p(_i32(token_seq, "token_seq")),
+          _p(_i32(block_table, "block_table")), block_table.shape[1], _p(k_pages), _p(v_pages), T, nh, nkv, hd, vd,
+          int(block_size), int(n_gate), coef, every, 1 if unit_values else 0, float(eps))
 
 
 def rmsnorm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
@@ -463,7 +538,8 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
          n_rows: int | None = None, n_out: int | None = None, up_offset: int = 0,
          norm: tuple | None = None, pair_ids: torch.Tensor | None = None, pair_div: int = 1,
          always: tuple | None = None, w_kblocked: bool = False, row_ss: tuple | None = None,
-         activation: str = "silu", store_activation: str | None = None) -> torch.Tensor:
+         activation: str = "silu", store_activation: str | None = None, activation_params: tuple = (0.0, 0.0),
+         pre_scale: torch.Tensor | None = None, pre_scale_rows: torch.Tensor | None = None) -> torch.Tensor:
     """C[m, n] = sum_k a[m, k] * w[n, k] with an epilogue.
 
     `w` is [N, K], or [E, N, K] with `expert_offsets` [E+1] (rows sorted by expert).
@@ -484,12 +560,17 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
     in (bfloat16 weights, EPI_STORE, at most 32 rows; see `can_fuse_norm`).
     `row_ss` = (ss [M, n] float32, eps): row m of the product is scaled by rsqrt(sum(ss[m]) / K + eps)
     before the bias is added (the rows of `a` are a ScaleLater's; plain stored bfloat16 product, M <= 64).
-    `store_activation` (one of STORED_ACTIVATIONS, EPI_STORE without bias): the product goes through it before it
-    is stored, e.g. "relu2" = max(x, 0)^2.
+    `store_activation` (one of STORED_ACTIVATIONS, EPI_STORE or EPI_STORE_F32 without bias): the product goes through
+    it before it is stored, e.g. "relu2" = max(x, 0)^2.
+    `activation_params` = (limit, alpha) for "swiglu_clamped": g = min(gate, limit), u = clamp(up, -limit, limit),
+    stored g sigmoid(alpha g) (u + 1).
+    `pre_scale` (EPI_GATED; float32): gate and up of logical row m are multiplied by pre_scale[m] (or by
+    pre_scale[pre_scale_rows[m]]) before the activation, which is what the activation sees when row m of `a` is
+    scaled by that number.
     """
     if store_activation not in STORED_ACTIVATIONS:
         raise KernelError(f"gemm: stored activation '{store_activation}' is not one of {sorted(k for k in STORED_ACTIVATIONS if k)}")
-    if store_activation is not None and (epilogue != EPI_STORE or bias is not None):
+    if store_activation is not None and (epilogue not in (EPI_STORE, EPI_STORE_F32) or bias is not None):
         raise KernelError("gemm: a stored activation goes with the plain stored product without bias")
     if row_ss is not None:
         ss = row_ss[0]
@@ -549,6 +630,11 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
         raise KernelError(f"gemm: output {tuple(out.shape)} {out.dtype} does not fit [{M},{N}] {out_dtype}")
     if bias is not None and bias.numel() != N:
         raise KernelError(f"gemm: bias has {bias.numel()} elements for {N} columns")
+    if pre_scale is not None:
+        if epilogue != EPI_GATED or pre_scale.dtype != torch.float32 or not pre_scale.is_contiguous() \
+                or (pre_scale_rows is None and pre_scale.numel() < M) or (pre_scale_rows is not None and pre_scale_rows.numel() < M):
+            raise KernelError("gemm: a scale in front of the activation is contiguous float32, one number per logical row, "
+                              "with the gate/up epilogue")
     _call("gemm", "fx_gemm", _stream(), dtype_code(w.dtype), epilogue, _p(a), a.stride(0), _p(w), w_stride, up_offset,
           _p(bias), dtype_code(bias.dtype) if bias is not None else 0, _p(out), out.stride(0),
           _p(row_scale), _p(_i32(a_rows, "a_rows")), _p(_i32(c_rows, "c_rows")),
@@ -558,7 +644,8 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
           _p(_i32(pair_ids, "pair_ids")), int(pair_div),
           n_always, always_rows, always_from_a, n_w if w_kblocked else 0,
           _p(row_ss[0]) if row_ss is not None else None, row_ss[0].shape[1] if row_ss is not None else 0,
-          ACTIVATIONS[activation], STORED_ACTIVATIONS[store_activation])
+          ACTIVATIONS[activation], STORED_ACTIVATIONS[store_activation], float(activation_params[0]),
+          float(activation_params[1]), _p(pre_scale), _p(_i32(pre_scale_rows, "pre_scale_rows")))
     return out
 
 
@@ -641,7 +728,7 @@ def attention_tile_queries(dtype, head_dim: int, block_size: int) -> int:
 def attention_tiles(q, out, k_pages, v_pages, block_table, positions, item_seq, item_tok, item_n,
                     n_heads, n_kv_heads, head_dim, block_size, window, scale, tile_q: int = 64, mask_chunk: int = 0,
                     v_dim: int | None = None, keep_first: int = 0, sinks=None, gate=None, softcap: float = 0.0,
-                    slopes=None) -> None:
+                    slopes=None, gate_per_head: bool = False) -> None:
     """Blocks of queries: item i is item_n[i] <= tile_q consecutive tokens of sequence item_seq[i] from token
     item_tok[i] on; tile_q is 64 or attention_tile_queries(...).  `mask_chunk` > 0: the chunked mask (a query sees
     the keys of its own chunk of that many positions) instead of a window.  `v_dim`: size of a value head where it
@@ -651,14 +738,14 @@ def attention_tiles(q, out, k_pages, v_pages, block_table, positions, item_seq, 
     `softcap` > 0: a scaled score s becomes softcap * tanh(s / softcap).  `slopes` (float32 [n_heads]): the score of
     key t for the query at position p then loses slopes[h] * (p - t)."""
     _check_attention_shapes(q, out, k_pages, v_pages, n_heads, n_kv_heads, head_dim, int(v_dim or head_dim), block_size)
-    _check_attention_extras(out, n_heads, int(v_dim or head_dim), window, keep_first, sinks, gate, softcap, slopes)
+    _check_attention_extras(out, n_heads, 1 if gate_per_head else int(v_dim or head_dim), window, keep_first, sinks, gate, softcap, slopes)
     _call("attention", "fx_attn_tiles", _stream(), dtype_code(q.dtype), _p(q), q.stride(0), _p(out), out.stride(0),
           _p(k_pages), _p(v_pages), _p(_i32(block_table, "block_table")), block_table.shape[1],
           _p(_i32(positions, "positions")), _p(_i32(item_seq, "item_seq")), _p(_i32(item_tok, "item_tok")),
           _p(_i32(item_n, "item_n")), item_seq.numel(), n_heads, n_kv_heads, head_dim, block_size,
           int(window or 0), float(scale), int(tile_q), int(v_dim or head_dim), int(mask_chunk or 0),
           int(keep_first or 0), _p(sinks), _p(gate), gate.stride(0) if gate is not None else 0, float(softcap or 0.0),
-          _p(slopes))
+          _p(slopes), 1 if gate_per_head else 0)
 
 
 def _check_attention_extras(out, n_heads, v_dim, window, keep_first, sinks, gate, softcap=0.0, slopes=None) -> None:
@@ -715,7 +802,7 @@ def decode_attention_chunk(n_items: int, n_heads: int, n_kv_heads: int, max_kv_l
 def attention_decode(q, out, k_pages, v_pages, block_table, positions, item_seq, item_tok,
                      n_heads, n_kv_heads, head_dim, block_size, window, scale, max_kv_len, chunk=None,
                      waves=0, mask_chunk: int = 0, v_dim: int | None = None, keep_first: int = 0, sinks=None,
-                     gate=None, softcap: float = 0.0, slopes=None) -> None:
+                     gate=None, softcap: float = 0.0, slopes=None, gate_per_head: bool = False) -> None:
     """Single queries.  The keys go to ceil(max_kv_len / chunk) blocks whose results are merged in ascending
     order.  float32 cuts them at multiples of `chunk`, 256 by default (so that a result does not depend on the
     batch); bfloat16, whose blocks of up to eight waves share a chunk, cuts every sequence's own range of keys (from
@@ -724,7 +811,7 @@ def attention_decode(q, out, k_pages, v_pages, block_table, positions, item_seq,
     n = item_seq.numel()
     v_dim = int(v_dim or head_dim)
     _check_attention_shapes(q, out, k_pages, v_pages, n_heads, n_kv_heads, head_dim, v_dim, block_size)
-    _check_attention_extras(out, n_heads, v_dim, window, keep_first, sinks, gate, softcap, slopes)
+    _check_attention_extras(out, n_heads, 1 if gate_per_head else v_dim, window, keep_first, sinks, gate, softcap, slopes)
     if chunk is None:
         chunk = 256
         if q.dtype == torch.bfloat16:
@@ -738,7 +825,7 @@ def attention_decode(q, out, k_pages, v_pages, block_table, positions, item_seq,
           n_heads, n_kv_heads, head_dim, block_size, int(window or 0), float(scale),
           _p(part_o), _p(part_ml), splits, chunk, int(waves), v_dim, int(mask_chunk or 0),
           int(keep_first or 0), _p(sinks), _p(gate), gate.stride(0) if gate is not None else 0, float(softcap or 0.0),
-          _p(slopes))
+          _p(slopes), 1 if gate_per_head else 0)
 
 
 def router_select(logits, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gate=False, selection_bias=None,
@@ -921,24 +1008,35 @@ def _f32_rows(t, what, cols):
     return t
 
 
-def short_conv(x, taps, state, token_seq, seq_starts, slot_ids, n_seqs: int) -> torch.Tensor:
-    """y[t, c] = silu(sum_j taps[c, n-1-j] x[t-j, c]) over each sequence's own tokens, the n-1 inputs from before
-    the step coming from state[slot, c, :] (oldest first), which afterwards holds the step's last n-1 inputs.
-    x: float32 [T, C] rows (any row stride); taps [C, n]; state float32 [slots, C, n-1]; sequence s owns tokens
-    [seq_starts[s], seq_starts[s+1]) and slot slot_ids[s].  Returns float32 [T, C]."""
+CONV_ACTIVATIONS = {None: 0, "silu": 1}
+
+
+def short_conv(x, taps, state, token_seq, seq_starts, slot_ids, n_seqs: int, activation: str | None = "silu", bias=None,
+               add_input: bool = False, out_dtype=torch.float32) -> torch.Tensor:
+    """y[t, c] = act(sum_j taps[c, n-1-j] x[t-j, c] (+ bias[c])) (+ x[t, c] with `add_input`) over each sequence's own
+    tokens, the n-1 inputs from before the step coming from state[slot, c, :] (oldest first), which afterwards holds
+    the step's last n-1 inputs.  x: float32 or bfloat16 [T, C] rows (any row stride); taps [C, n] (and bias [C] of
+    the taps' type); state float32 [slots, C, n-1]; sequence s owns tokens [seq_starts[s], seq_starts[s+1]) and slot
+    slot_ids[s]; `activation` None or "silu".  Returns [T, C] in `out_dtype` (float32, or x's type); the sums are float32."""
     T, C = x.shape
     n = taps.shape[1]
-    _f32_rows(x, "short_conv: x", C)
+    if activation not in CONV_ACTIVATIONS:
+        raise KernelError(f"short_conv: activation '{activation}' is not one of {list(CONV_ACTIVATIONS)}")
+    if x.dim() != 2 or x.stride(1) != 1 or out_dtype not in (torch.float32, x.dtype):
+        raise KernelError("short_conv: x must be rows with unit inner stride, the output float32 or of x's type")
+    if bias is not None and (bias.numel() != C or bias.dtype != taps.dtype or not bias.is_contiguous()):
+        raise KernelError(f"short_conv: bias of {bias.numel()} elements ({bias.dtype}) for {C} channels of {taps.dtype} taps")
     if tuple(taps.shape) != (C, n) or not taps.is_contiguous():
         raise KernelError(f"short_conv: taps {tuple(taps.shape)} for {C} channels")
     if state.dtype != torch.float32 or not state.is_contiguous() or tuple(state.shape[1:]) != (C, max(n - 1, 0)):
         raise KernelError(f"short_conv: state {tuple(state.shape)} for [slots, {C}, {n - 1}]")
     if seq_starts.numel() < n_seqs + 1 or slot_ids.numel() < n_seqs or token_seq.numel() < T:
         raise KernelError("short_conv: the step's index tensors are shorter than its sequences and tokens")
-    y = torch.empty((T, C), dtype=torch.float32, device=x.device)
-    _call("recurrent", "fx_short_conv", _stream(), _p(x), x.stride(0), _p(y), y.stride(0), _p(taps), dtype_code(taps.dtype), n,
+    y = torch.empty((T, C), dtype=out_dtype, device=x.device)
+    _call("recurrent", "fx_short_conv", _stream(), _p(x), dtype_code(x.dtype), x.stride(0), _p(y), dtype_code(out_dtype),
+          y.stride(0), _p(taps), dtype_code(taps.dtype), n,
           _p(state), _p(_i32(token_seq, "token_seq")), _p(_i32(seq_starts, "seq_starts")), _p(_i32(slot_ids, "slot_ids")),
-          T, int(n_seqs), C)
+          T, int(n_seqs), C, _p(bias), CONV_ACTIVATIONS[activation], 1 if add_input else 0)
     return y
 
 
@@ -991,19 +1089,111 @@ def channel_delta(qn, kn, decay, beta, kq, v, state, seq_starts, slot_ids, n_seq
 HEAD_GATES = {"sigmoid": 0, "silu": 1}
 
 
-def gated_head_norm(o, gate, weight, eps: float, n_heads: int, v_dim: int, out_dtype, gate_activation: str = "sigmoid") -> torch.Tensor:
+def gated_head_norm(o, gate, weight, eps: float, n_heads: int, v_dim: int, out_dtype, gate_activation: str = "sigmoid",
+                    denominators: tuple | None = None) -> torch.Tensor:
     """y[t, h, :] = o[t, h, :] / rms(o[t, h, :]) * weight * act(gate[t, h, :]) in `out_dtype`, act being sigmoid or
-    silu; o and gate are float32 rows [T, H*V], weight [V] is shared by the heads."""
+    silu; o and gate are float32 rows [T, H*V]; weight is [V], shared by the heads, or [H*V], one per head and channel.
+    `denominators` = (nq, m), float32 [T, H] each: o[t, h] is first divided by max(|nq|, exp(-m)) + 1e-6."""
     if gate_activation not in HEAD_GATES:
         raise KernelError(f"gated_head_norm: gate activation '{gate_activation}' is not one of {sorted(HEAD_GATES)}")
     T = o.shape[0]
     H, V = int(n_heads), int(v_dim)
     _f32_rows(o, "gated_head_norm: o", H * V), _f32_rows(gate, "gated_head_norm: gate", H * V)
-    if gate.shape[0] != T or weight.numel() != V or not weight.is_contiguous():
+    if gate.shape[0] != T or weight.numel() not in (V, H * V) or not weight.is_contiguous():
         raise KernelError(f"gated_head_norm: gate {tuple(gate.shape)} / weight {tuple(weight.shape)} for {T} x {H} heads of {V}")
+    nq = m = None
+    if denominators is not None:
+        nq, m = denominators
+        for t in (nq, m):
+            if t.dtype != torch.float32 or not t.is_contiguous() or tuple(t.shape) != (T, H):
+                raise KernelError(f"gated_head_norm: denominators must be contiguous float32 [{T}, {H}]")
     y = torch.empty((T, H * V), dtype=out_dtype, device=o.device)
     _call("recurrent", "fx_gated_head_norm", _stream(), dtype_code(out_dtype), _p(o), o.stride(0), _p(gate), gate.stride(0),
-          _p(weight), dtype_code(weight.dtype), _p(y), y.stride(0), T, H, V, float(eps), HEAD_GATES[gate_activation])
+          _p(weight), dtype_code(weight.dtype), 1 if (weight.numel() == H * V and H > 1) else 0, _p(y), y.stride(0), T, H, V,
+          float(eps), HEAD_GATES[gate_activation], _p(nq), _p(m))
+    return y
+
+
+def gated_outer(q, k, v, keep, take, state, seq_starts, slot_ids, n_seqs: int, n_heads: int, n_kv_heads: int, key_dim: int,
+                v_dim: int, q_scale: float = 1.0, normalizer: bool = False):
+    """A matrix memory with one forgetting and one writing factor per head and token, over each sequence's tokens in
+    order, from and into state[slot]:  S <- keep_t S + take_t k_t v_t^T;  o_t = q_scale S^T q_t.  q, k: float32 rows
+    [T, G*D]; v [T, H*V]; `keep` float32 [T, H], or [H] (the same factors at every token); `take` float32 [T, H] or
+    None (1).  The state is float32 [slots, H, V, D] (transposed).  With `normalizer` it is [slots, H, V + 1, D]: its
+    last column is n <- keep_t n + take_t k_t, and the call also returns nq [T, H] = q_scale n_t . q_t.
+    Returns o float32 [T, H*V], or (o, nq)."""
+    T = q.shape[0]
+    H, G, D, V = int(n_heads), int(n_kv_heads), int(key_dim), int(v_dim)
+    _f32_rows(q, "gated_outer: q", G * D), _f32_rows(k, "gated_outer: k", G * D), _f32_rows(v, "gated_outer: v", H * V)
+    keep_const = keep.dim() == 1
+    if keep.dtype != torch.float32 or not keep.is_contiguous() or tuple(keep.shape) not in ((H,), (T, H)):
+        raise KernelError(f"gated_outer: forgetting factors {tuple(keep.shape)} for [{T}, {H}] or [{H}]")
+    if take is not None and (take.dtype != torch.float32 or not take.is_contiguous() or tuple(take.shape) != (T, H)):
+        raise KernelError(f"gated_outer: writing factors must be contiguous float32 [{T}, {H}]")
+    VS = V + (1 if normalizer else 0)
+    if k.shape[0] != T or v.shape[0] != T or state.dtype != torch.float32 or not state.is_contiguous() \
+            or tuple(state.shape[1:]) != (H, VS, D):
+        raise KernelError(f"gated_outer: k {tuple(k.shape)} / v {tuple(v.shape)} / state {tuple(state.shape)} for [slots, {H}, {VS}, {D}]")
+    if seq_starts.numel() < n_seqs + 1 or slot_ids.numel() < n_seqs:
+        raise KernelError("gated_outer: the step's index tensors are shorter than its sequences")
+    out = torch.empty((T, H * V), dtype=torch.float32, device=q.device)
+    nq = torch.empty((T, H), dtype=torch.float32, device=q.device) if normalizer else None
+    _call("recurrent", "fx_gated_outer", _stream(), _p(q), q.stride(0), _p(k), k.stride(0), _p(v), v.stride(0), _p(keep),
+          1 if keep_const else 0, _p(take), _p(out), out.stride(0), _p(nq), _p(state), _p(_i32(seq_starts, "seq_starts")),
+          _p(_i32(slot_ids, "slot_ids")), int(n_seqs), H, G, D, V, float(q_scale))
+    return (out, nq) if normalizer else out
+
+
+def exp_gate_scan(x_in, x_forget, cap: float, state, seq_starts, slot_ids, n_seqs: int, n_heads: int):
+    """Exponential gates under a running maximum, per head over each sequence's tokens in order.  From the float32
+    rows x_in, x_forget [T, H]:  i = cap tanh(x_in / cap);  f = logsigmoid(cap tanh(x_forget / cap));
+    m_t = max(f + m_(t-1), i);  keep_t = exp(f + m_(t-1) - m_t);  take_t = exp(i - m_t).  m is carried in
+    state [slots, H] (float32).  Returns (keep, take, m), float32 [T, H] each."""
+    T, H = x_in.shape[0], int(n_heads)
+    _f32_rows(x_in, "exp_gate_scan: x_in", H), _f32_rows(x_forget, "exp_gate_scan: x_forget", H)
+    if x_forget.shape[0] != T or state.dtype != torch.float32 or not state.is_contiguous() or tuple(state.shape[1:]) != (H,):
+        raise KernelError(f"exp_gate_scan: state {tuple(state.shape)} for [slots, {H}]")
+    if seq_starts.numel() < n_seqs + 1 or slot_ids.numel() < n_seqs:
+        raise KernelError("exp_gate_scan: the step's index tensors are shorter than its sequences")
+    keep, take, m = (torch.empty((T, H), dtype=torch.float32, device=x_in.device) for _ in range(3))
+    _call("recurrent", "fx_exp_gate_scan", _stream(), _p(x_in), x_in.stride(0), _p(x_forget), x_forget.stride(0), float(cap),
+          _p(keep), _p(take), _p(m), _p(state), _p(_i32(seq_starts, "seq_starts")), _p(_i32(slot_ids, "slot_ids")),
+          int(n_seqs), H)
+    return keep, take, m
+
+
+def rglru(u, gate_logits, gate_bias, n_parts: int, lam, branch, state, seq_starts, slot_ids, n_seqs: int, longest: int,
+          out_dtype, rate: float = 8.0) -> torch.Tensor:
+    """The real-gated linear recurrent unit per channel, over each sequence's tokens in order, from and into
+    state[slot] (float32 [slots, C]):  a = exp(-rate sigmoid(r) softplus(lam));
+    S_t = a_t S_(t-1) + sqrt(1 - a_t^2) sigmoid(i) u_t;  y_t = S_t gelu_tanh(branch_t).  u, branch: float32 rows
+    [T, C]; lam [C].  The gates' logits r and i come as the products of the channels' `n_parts` parts leave them:
+    gate_logits contiguous float32 [T, n_parts, 2, C / n_parts] (recurrence gate, then input gate), plus gate_bias
+    of shape [n_parts, 2, C / n_parts] (or None).  `longest`: the most tokens a sequence of the step brings (it picks
+    how a sequence's tokens are dealt out to waves).  Returns y [T, C] in `out_dtype`."""
+    T, C = u.shape
+    for t, what in ((u, "u"), (branch, "branch")):
+        _f32_rows(t, f"rglru: {what}", C)
+        if t.shape[0] != T:
+            raise KernelError(f"rglru: {what} has {t.shape[0]} rows, u {T}")
+    if n_parts < 1 or C % n_parts or gate_logits.dtype != torch.float32 or not gate_logits.is_contiguous() \
+            or gate_logits.numel() != 2 * T * C:
+        raise KernelError(f"rglru: gate logits {tuple(gate_logits.shape)} for {T} tokens, {n_parts} parts of {C} channels")
+    if gate_bias is not None and (gate_bias.dtype != torch.float32 or not gate_bias.is_contiguous() or gate_bias.numel() != 2 * C):
+        raise KernelError(f"rglru: the gates' bias must hold {2 * C} contiguous float32 values")
+    if lam.numel() != C or not lam.is_contiguous() or state.dtype != torch.float32 or not state.is_contiguous() \
+            or tuple(state.shape[1:]) != (C,):
+        raise KernelError(f"rglru: lam {tuple(lam.shape)} / state {tuple(state.shape)} for {C} channels")
+    if seq_starts.numel() < n_seqs + 1 or slot_ids.numel() < n_seqs:
+        raise KernelError("rglru: the step's index tensors are shorter than its sequences")
+    a = torch.empty((T, C), dtype=torch.float32, device=u.device)
+    x = torch.empty((T, C), dtype=torch.float32, device=u.device)
+    _call("recurrent", "fx_rglru_gates", _stream(), _p(u), u.stride(0), _p(gate_logits), _p(gate_bias), _p(lam),
+          dtype_code(lam.dtype), float(rate), _p(a), _p(x), T, C, int(n_parts))
+    y = torch.empty((T, C), dtype=out_dtype, device=u.device)
+    _call("recurrent", "fx_rglru_scan", _stream(), dtype_code(out_dtype), _p(a), _p(x), _p(branch), branch.stride(0), _p(y),
+          y.stride(0), _p(state), _p(_i32(seq_starts, "seq_starts")), _p(_i32(slot_ids, "slot_ids")), int(n_seqs), C,
+          int(longest))
     return y
 
 

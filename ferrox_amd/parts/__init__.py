@@ -1,4 +1,4 @@
-from . import attention, block, composite, embedding, latent, mlp, moe, norm, recurrent, rope  # noqa: F401  (registration)
+from . import attention, block, composite, embedding, gated_linear, latent, mlp, moe, norm, recurrent, rope  # noqa: F401  (registration)
 from .base import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSITION_ENCODINGS, Block,
                    FeedForward, LayerCache, LayerSpec, Mixer, ModelSpec, Norm, ParamSpec, Part, PartSpec,
                    PositionEncoding, Rotary, ScheduleEntry, StepContext, walk_params, walk_parts)

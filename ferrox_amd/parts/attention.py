@@ -71,7 +71,8 @@ class PagedAttention(Mixer):
                  qk_norm: PartSpec | None = None, v_dim: int | None = None, chunk: int | None = None,
                  names: dict | None = None, keep_first: int = 0, sink: bool = False, out_gate: bool = False,
                  own_kv: bool = True, retain: tuple | None = None, softcap: float | None = None,
-                 distance_slopes=None, values_from_keys: bool = False, qk_norm_span: str = "head"):
+                 distance_slopes=None, values_from_keys: bool = False, qk_norm_span: str = "head",
+                 q_temperature: tuple | None = None, unit_values: float | None = None):
         """`qk_norm`: kind and arguments of a norm over head_dim; two of them are built, with tensors under
         `q_norm.` and `k_norm.`, and applied to every head of q and of k before the rotation.
         `v_dim`: size of a value head where it differs from head_dim (the size of a query and key head).
@@ -82,7 +83,11 @@ class PagedAttention(Mixer):
         `keep_first` (with a window): the first so many keys of a sequence stay visible to every later query.
         `sink`: a learned logit per head ([n_heads]) joins the softmax's denominator; it has no key and no value.
         `out_gate`: the heads' outputs are multiplied by sigmoid(W_g x), x the mixer's input, before the output
-        projection (W_g: [n_heads * v_dim, hidden]).
+        projection (W_g: [n_heads * v_dim, hidden]); "head": one gate per head, W_g: [n_heads, hidden].
+        `q_temperature` = (coef, every): the query at position p is multiplied by 1 + coef ln(floor((p + 1) / every) + 1),
+        which is how positions enter the scores of such a mixer (it rotates nothing).
+        `unit_values` (an eps): every value head is divided by its root mean square over v_dim (eps inside the root,
+        no weight) and cached so.
         `own_kv` False: the mixer has no key and value projections and writes no cache; its schedule entry reads
         the cache of an entry that has them (with these head counts and sizes).
         `retain` = (window or None, keep_first): how the pages of this mixer's cache group age, where that is not
@@ -108,6 +113,16 @@ class PagedAttention(Mixer):
         if self.keep_first < 0:
             raise ValueError(f"keep_first {keep_first} is negative")
         self.has_sink, self.out_gate, self.own_kv = bool(sink), bool(out_gate), bool(own_kv)
+        self.gate_per_head = out_gate == "head"
+        self.q_temperature = (float(q_temperature[0]), int(q_temperature[1])) if q_temperature else None
+        if self.q_temperature and self.q_temperature[1] < 1:
+            raise ValueError(f"a query temperature that steps every {q_temperature[1]} positions")
+        self.unit_values = float(unit_values) if unit_values is not None else None
+        # queries warmed by position or values of unit size: both are float32 arithmetic on the products' float32 rows,
+        # done by the launch that writes the cache
+        self.prepares = self.q_temperature is not None or self.unit_values is not None
+        if self.prepares and (bias or qk_norm is not None or values_from_keys or not own_kv):
+            raise ValueError("a query temperature and unit values go with projections of q, k and v without biases and head norms")
         if self.chunk and (retain is not None or keep_first):
             raise ValueError("kept first keys and a retention of their own go with a window, not with a chunked mask")
         # (None, 0): every key is kept; (W, F): the last W and the first F
@@ -156,6 +171,8 @@ class PagedAttention(Mixer):
                 raise ValueError("norms over the whole projection are RMS norms with a weight, under a mixer that rotates nothing")
         elif qk_norm is not None:
             self.q_norm, self.k_norm = (NORMS.build(PartSpec(qk_norm.kind, dict(qk_norm.args))) for _ in range(2))
+        if self.prepares and (self.position.rotary() is None or self.position.rotary().rotary_dim):
+            raise ValueError("a query temperature and unit values go with a mixer that rotates nothing")
         if (self.position.rotary() or Rotary(0, 1.0)).magnitude != 1.0:
             raise ValueError("this mixer's rotation kernels turn and do not stretch: a rotation's magnitude must be 1")
         if bias and out_gate:
@@ -178,7 +195,7 @@ class PagedAttention(Mixer):
         if self.has_sink:
             specs[n["sink"]] = ParamSpec((self.n_heads,))
         if self.out_gate:
-            specs[n["gate"]] = ParamSpec((self.ow, H))
+            specs[n["gate"]] = ParamSpec((self.n_heads if self.gate_per_head else self.ow, H))
         return specs
 
     def load(self, fetch):
@@ -237,7 +254,7 @@ class PagedAttention(Mixer):
         # (heads that are normed again take their q and k from a float32 product; the norm inside two products, one
         # of them stored in float32, was measured and is behind the norm kernel: every block norms all rows)
         if (ctx.act_dtype != torch.bfloat16 or rms is None or residual.shape[0] > 16 or self.q_norm is not None
-                or not self.own_kv or not ops.can_fuse_norm(residual, self.qkv.weight, residual.shape[0])):
+                or self.prepares or not self.own_kv or not ops.can_fuse_norm(residual, self.qkv.weight, residual.shape[0])):
             return False
         debug.region("qkv")
         qkv = ops.gemm(residual, self.qkv.weight, bias=self.qkv.bias, norm=rms)
@@ -247,7 +264,7 @@ class PagedAttention(Mixer):
     def takes_scale_later(self, act_dtype) -> bool:
         """Whether forward takes an ops.ScaleLater as x (the block before then leaves its rows that way)."""
         w = self.qkv.weight
-        return (self.q_norm is None and self.own_kv and act_dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+        return (self.q_norm is None and not self.prepares and self.own_kv and act_dtype == torch.bfloat16 and w.dtype == torch.bfloat16
                 and w.shape[1] % 8 == 0 and w.data_ptr() % 16 == 0)
 
     def tile_queries(self, ctx, dtype, block_size: int) -> int:
@@ -334,7 +351,7 @@ class PagedAttention(Mixer):
         k_pages, v_pages = cache.pages["k"], cache.pages["v"]
         rot = self.position.rotary()
         debug.region("qkv")
-        fused = (qkv is None and self.q_norm is None and rot is not None and rot.frequencies is None
+        fused = (qkv is None and self.q_norm is None and rot is not None and rot.frequencies is None and not self.prepares
                  and self.v_dim == self.head_dim and self.own_kv and not self.out_gate
                  and ops.can_qkv_rope(x, self.qkv.weight, ctx.n_tokens, self.head_dim, rot.rotary_dim, rot.interleaved))
         if fused:
@@ -347,7 +364,21 @@ class PagedAttention(Mixer):
         else:
             gate = None
             wrote = False
-            if self.q_norm is not None:           # every head of q and k through its norm, between bias and rotation
+            if self.prepares:
+                # one float32 product, then one launch: q times its position's temperature, the gate's columns behind
+                # it, k into its page, v (of unit size) into its page
+                n_gate = (self.n_heads if self.gate_per_head else self.ow) if self.out_gate else 0
+                rows = matmul(x, self.qkv.weight, epilogue=ops.EPI_STORE_F32)
+                qkv = torch.empty((ctx.n_tokens, self.qw + n_gate), dtype=ctx.act_dtype, device=rows.device)
+                debug.region("rope + cache write")
+                ops.temp_unit_kv_write(rows, qkv, ctx.positions, ctx.token_seq, table, k_pages if cache.writes else None,
+                                       v_pages if cache.writes else None, self.n_heads, self.n_kv_heads, self.head_dim,
+                                       self.v_dim, cache.block_size, n_gate=n_gate, temperature=self.q_temperature,
+                                       unit_values=self.unit_values is not None, eps=self.unit_values or 0.0)
+                q, k, v, wrote = qkv[:, :self.qw], None, None, True
+                if n_gate:
+                    gate = qkv[:, self.qw:]
+            elif self.q_norm is not None:           # every head of q and k through its norm, between bias and rotation
                 if self.span_norms:
                     q, rest = self.normed_spans_and_cache(x, ctx, table, cache)
                     k, wrote = None, True
@@ -388,7 +419,8 @@ class PagedAttention(Mixer):
         common = (self.n_heads, self.n_kv_heads, self.head_dim, cache.block_size, self.window, self.scale)
         # (the gate multiplies the heads' outputs as the attention kernels write them)
         mask = dict(mask_chunk=self.chunk or 0, v_dim=self.v_dim, keep_first=self.keep_first, sinks=self.sinks,
-                    gate=None if fused else gate, softcap=self.softcap, slopes=self.slopes)
+                    gate=None if fused else gate, softcap=self.softcap, slopes=self.slopes,
+                    gate_per_head=self.gate_per_head and gate is not None)
         if items["n_tiles"]:
             ops.attention_tiles(q, out, k_pages, v_pages, table, ctx.positions,
                                 items["tile_seq"], items["tile_tok"], items["tile_n"], *common, tile_q=tile_q, **mask)

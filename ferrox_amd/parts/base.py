@@ -19,7 +19,7 @@ Interfaces (all tensors on the GPU; `h` is the float32 residual stream [T, H],
                    cache_group() -> (key, window), state_shapes() -> {name: (shape, dtype)}, graph_safe,
                    forward(x, ctx, cache, residual) -> None   (adds its output into residual)
   FeedForward      forward(x, ctx, residual) -> None
-  Block            forward(h, ctx, cache) -> None
+  Block            forward(h, ctx, cache) -> None, state_shapes() -> {name: (shape, dtype)} (what the block itself carries)
   every part       param_specs() -> {local name: ParamSpec}, load(fetch), kernel_libraries;
                    borrows() -> [full names of tensors that other parts own and this one reads too]
 """
@@ -53,6 +53,7 @@ class LayerSpec:
     block: str                # kind of block, e.g. 'prenorm'
     prefix: str               # e.g. 'model.layers.3.'
     parts: dict               # slot name -> PartSpec
+    args: dict = field(default_factory=dict)     # what the block itself is built with beside its parts (sizes, tensor names)
 
 
 @dataclass(frozen=True)
@@ -311,6 +312,11 @@ class Block(Part):
 
     def takes_scale_later(self, act_dtype) -> bool:
         return False
+
+    def state_shapes(self) -> dict:
+        """State that the block itself carries from step to step for every request, beside its mixer's:
+        name -> (shape, dtype).  It lies in the request's slot under `block.<name>` of the layer's cache."""
+        return {}
 
     def forward(self, h, ctx: StepContext, cache: LayerCache) -> None:
         raise NotImplementedError

@@ -4,7 +4,8 @@ from __future__ import annotations
 import torch
 
 from .. import debug
-from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Block
+from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Block, ParamSpec
+from .linear import Linear
 
 
 @BLOCKS.register("prenorm")
@@ -123,3 +124,89 @@ class ParallelBlock(Block):
         self.mixer.forward(x, ctx, cache, h)
         if self.ffn is not None:
             self.ffn.forward(x, ctx, h)
+
+
+@BLOCKS.register("gated_prenorm")
+class GatedPreNormBlock(Block):
+    """h += G1 * mixer(C(x1)),  x1 = norm1(h);  h += G2 * ffn(x2),  x2 = norm2(h), with two optional additions to the
+    pre-norm block:
+      * an input convolution, C(x) = x + conv(x): a short causal convolution over time on each channel of what the
+        mixer reads (`conv_taps` >= 1; weights [hidden, taps], the last column meets the current token; no bias, no
+        activation).  The last taps - 1 normed rows of every request are part of its state (`block.conv`).
+      * a gated residual, G = sigmoid(W x + b) element by element, x being the normed rows the sublayer was handed
+        (before the input convolution): a sublayer's float32 output rows pass the gate as they join the stream.
+    A layer without a feed-forward has the first half only.  The sublayers add into a zeroed float32 buffer in
+    place of the stream (their last product's epilogue), which one kernel then gates and adds."""
+    slots = {"norm1": NORMS, "mixer": MIXERS, "norm2": NORMS, "ffn": FEED_FORWARDS}
+    optional_slots = ("norm2", "ffn")
+    kernel_libraries = ("elementwise", "gemm", "recurrent")
+    TENSORS = {"conv": "conv1", "gate1": "gate1.weight", "gate1_bias": "gate1.bias", "gate2": "gate2.weight",
+               "gate2_bias": "gate2.bias"}
+
+    def __init__(self, parts: dict, prefixes: dict, hidden_size: int, conv_taps: int = 0, residual_gates: bool = True,
+                 names: dict | None = None):
+        self.norm1, self.mixer, self.norm2, self.ffn = parts["norm1"], parts["mixer"], parts.get("norm2"), parts.get("ffn")
+        if (self.ffn is None) != (self.norm2 is None):
+            raise ValueError("a gated pre-norm block has a feed-forward and its norm, or neither")
+        self.hidden_size, self.conv_taps, self.residual_gates = int(hidden_size), int(conv_taps or 0), bool(residual_gates)
+        if self.conv_taps > 16:
+            raise ValueError(f"conv_taps {conv_taps}: the convolution kernel takes up to 16 taps")
+        self.names = dict(self.TENSORS, **(names or {}))
+        self._prefixes = prefixes
+        self.taps = self.gate1 = self.gate2 = None
+
+    def children(self):
+        return [(self._prefixes[s], getattr(self, s)) for s in ("norm1", "mixer", "norm2", "ffn") if getattr(self, s) is not None]
+
+    def param_specs(self):
+        W, n = self.hidden_size, self.names
+        specs = {}
+        if self.conv_taps:
+            specs[n["conv"]] = ParamSpec((W, self.conv_taps))
+        if self.residual_gates:
+            specs.update({n["gate1"]: ParamSpec((W, W)), n["gate1_bias"]: ParamSpec((W,), init="zeros")})
+            if self.ffn is not None:
+                specs.update({n["gate2"]: ParamSpec((W, W)), n["gate2_bias"]: ParamSpec((W,), init="zeros")})
+        return specs
+
+    def load(self, fetch):
+        n = self.names
+        if self.conv_taps:
+            self.taps = fetch(n["conv"]).float().contiguous()
+        if self.residual_gates:
+            self.gate1 = Linear(fetch(n["gate1"]), fetch(n["gate1_bias"]).float().contiguous())
+            if self.ffn is not None:
+                self.gate2 = Linear(fetch(n["gate2"]), fetch(n["gate2_bias"]).float().contiguous())
+
+    def state_shapes(self) -> dict:
+        return {"conv": ((self.hidden_size, self.conv_taps - 1), torch.float32)} if self.conv_taps else {}
+
+    def _join(self, h, out, gate, x):
+        from .. import ops
+        debug.region("residual gate")
+        if gate is None:
+            ops.residual_add(h, out)
+        else:
+            ops.gated_add(h, out, gate(x, epilogue=ops.EPI_STORE_F32))
+
+    def forward(self, h, ctx, cache):
+        from .. import ops
+        from .recurrent import sequence_starts
+        debug.region("norm")
+        x = self.norm1.forward(h, ctx)
+        read = x
+        if self.conv_taps:
+            debug.region("input conv")
+            read = ops.short_conv(x, self.taps, cache.state["block.conv"], ctx.token_seq, sequence_starts(ctx), ctx.slot_ids,
+                                  ctx.n_seqs, activation=None, add_input=True, out_dtype=x.dtype)
+        out = torch.empty_like(h)
+        ops.fill_u32(out, 0)
+        self.mixer.forward(read, ctx, cache, out)
+        self._join(h, out, self.gate1, x)
+        if self.ffn is None:
+            return
+        debug.region("norm")
+        x = self.norm2.forward(h, ctx)
+        ops.fill_u32(out, 0)
+        self.ffn.forward(x, ctx, out)
+        self._join(h, out, self.gate2, x)

@@ -15,22 +15,36 @@ from .linear import matmul
 class TokenEmbedding(Part):
     kernel_libraries = ("elementwise",)
 
-    def __init__(self, vocab_size: int, hidden_size: int, name: str = "weight", scale: float = 1.0):
-        """`scale`: a constant that every embedding row is multiplied by on its way into the float32 stream."""
+    def __init__(self, vocab_size: int, hidden_size: int, name: str = "weight", scale: float = 1.0,
+                 position_table: str | None = None, max_positions: int = 0):
+        """`scale`: a constant that every embedding row is multiplied by on its way into the float32 stream.
+        `position_table`: the name of a learned [max_positions, hidden] table; row p of it is added (unscaled) to
+        the row of a token at position p."""
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.name = name
         self.scale = float(scale)
         if not math.isfinite(self.scale):
             raise ValueError(f"an embedding scale of {scale}")
-        self.weight = None
+        self.position_table, self.max_positions = position_table or None, int(max_positions)
+        if self.position_table and self.max_positions < 1:
+            raise ValueError("a table of positions needs `max_positions`")
+        self.uses_positions = self.position_table is not None       # forward then takes positions=
+        self.weight = self.positions = None
 
     def param_specs(self):
-        return {self.name: ParamSpec((self.vocab_size, self.hidden_size))}
+        specs = {self.name: ParamSpec((self.vocab_size, self.hidden_size))}
+        if self.position_table:
+            specs[self.position_table] = ParamSpec((self.max_positions, self.hidden_size))
+        return specs
 
     def load(self, fetch):
         self.weight = fetch(self.name).contiguous()
+        if self.position_table:
+            self.positions = fetch(self.position_table).to(self.weight.dtype).contiguous()
 
-    def forward(self, token_ids):
+    def forward(self, token_ids, positions=None):
+        if self.position_table:
+            return ops.embed(self.weight, token_ids, scale=self.scale, position_table=self.positions, positions=positions)
         return ops.embed(self.weight, token_ids, scale=self.scale)
 
 

@@ -44,11 +44,14 @@ class SparseMoE(FeedForward):
     def __init__(self, hidden_size: int, n_experts: int, top_k: int, expert_intermediate_size: int,
                  norm_topk_prob: bool, gating: str = "softmax", shared_intermediate_size: int = 0,
                  shared_gate: bool = True, activation: str = "silu", weight_scale: float = 1.0, renorm_eps: float = 0.0,
-                 names: dict | None = None):
+                 names: dict | None = None, activation_params: tuple = (0.0, 0.0), weight_input: bool = False):
         """`weight_scale`: a constant that every mixture weight is multiplied by.  `renorm_eps`: added to the sum of the
         chosen scores before the weights are divided by it (with `norm_topk_prob`).  `names`: what the checkpoint calls
         this part's tensors, where that differs from `TENSORS` ('{}' stands for an expert's number; `shared` is the
-        shared expert's prefix and `shared_names` its own three names)."""
+        shared expert's prefix and `shared_names` its own three names).  `activation_params`: (limit, alpha) of the
+        "swiglu_clamped" gate.  `weight_input`: a chosen expert's weight multiplies the row that the expert reads, not
+        what it returns (the experts' outputs are then summed as they are); the gate/up product applies it to its sums
+        in front of the activation, which is the same number up to rounding."""
         if not 1 <= top_k <= n_experts:
             raise ValueError(f"top_k {top_k} must lie in 1..{n_experts}")
         if n_experts > limits.MOE_MAX_EXPERTS or top_k > limits.MOE_MAX_TOP_K:
@@ -59,6 +62,10 @@ class SparseMoE(FeedForward):
         if activation not in ops.ACTIVATIONS:
             raise ValueError(f"activation '{activation}' is not one of {sorted(ops.ACTIVATIONS)}")
         self.activation = activation
+        self.activation_params = (float(activation_params[0]), float(activation_params[1]))
+        self.weight_input = bool(weight_input)
+        if self.weight_input and shared_intermediate_size > 0:
+            raise ValueError("weights on the experts' input and a shared expert have no kernel together")
         self.hidden_size, self.n_experts, self.top_k = int(hidden_size), int(n_experts), int(top_k)
         self.expert_intermediate_size = int(expert_intermediate_size)
         self.norm_topk_prob, self.gating = bool(norm_topk_prob), GATINGS[gating]
@@ -117,6 +124,20 @@ class SparseMoE(FeedForward):
             router = torch.cat(same_dtype([router, fetch(n["shared_gate"]).reshape(1, -1)]), dim=0)
         self.router = router.contiguous()
 
+    def _gated(self, weights, order=None) -> dict:
+        """What the gate/up product is told beside its operands: the activation, and, where the weights act on the
+        experts' input, the weights as a scale in front of it (`order`: the pair that each sorted row stands for)."""
+        kw = dict(activation=self.activation, activation_params=self.activation_params)
+        if self.weight_input:
+            kw.update(pre_scale=weights.reshape(-1), pre_scale_rows=order)
+        return kw
+
+    def _mix(self, weights):
+        """The weights of the combine: ones where the weights have acted on the experts' input already."""
+        if not self.weight_input:
+            return weights
+        return ops.constant_rows(weights.device, 1.0, weights.numel()).view(weights.shape)
+
     @staticmethod
     def _then(then_norm, ctx, n_tokens) -> dict:
         """How the combine prepares the new rows for the next block's norm: `then_norm` is (norm, whether the
@@ -172,8 +193,8 @@ class SparseMoE(FeedForward):
             S, n = sorted_pieces, ids.numel()
             kb = dict(w_kblocked=True) if self.kblocked else {}
             debug.region("experts gate/up")
-            act = matmul(x, self.w_gate_up_all, epilogue=ops.EPI_GATED, activation=self.activation, a_rows=sorted_token, expert_offsets=offsets,
-                         n_rows=n + S * T, **kb)
+            act = matmul(x, self.w_gate_up_all, epilogue=ops.EPI_GATED, a_rows=sorted_token, expert_offsets=offsets,
+                         n_rows=n + S * T, **self._gated(weights, sorted_pair), **kb)
             debug.region("experts down")
             y = matmul(act, self.w_down_all, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets, c_rows=sorted_pair, **kb)
             debug.region("combine")
@@ -187,8 +208,8 @@ class SparseMoE(FeedForward):
                 debug.routing_trace.put(ids)
             S, n = self.shared_pieces, ids.numel()
             debug.region("experts gate/up")
-            act = ops.gemm(x, self.w_gate_up_all, epilogue=ops.EPI_GATED, activation=self.activation, pair_ids=ids, pair_div=self.top_k,
-                           always=(S, T, True), w_kblocked=self.kblocked)
+            act = ops.gemm(x, self.w_gate_up_all, epilogue=ops.EPI_GATED, pair_ids=ids, pair_div=self.top_k,
+                           always=(S, T, True), w_kblocked=self.kblocked, **self._gated(weights))
             debug.region("experts down")
             y = ops.gemm(act, self.w_down_all, epilogue=ops.EPI_STORE_F32, pair_ids=ids, always=(S, T, False),
                          w_kblocked=self.kblocked)
@@ -241,12 +262,12 @@ class SparseMoE(FeedForward):
         kb = dict(w_kblocked=True) if self.kblocked else {}
         debug.region("experts gate/up")
         if offsets is None:      # few pairs, unsorted: row p of `act` and of `y` is pair p
-            act = ops.gemm(x, self.w_gate_up, epilogue=ops.EPI_GATED, activation=self.activation, pair_ids=ids, pair_div=self.top_k, **kb)
+            act = ops.gemm(x, self.w_gate_up, epilogue=ops.EPI_GATED, pair_ids=ids, pair_div=self.top_k, **self._gated(weights), **kb)
             debug.region("experts down")
             y = ops.gemm(act, self.w_down, epilogue=ops.EPI_STORE_F32, pair_ids=ids, **kb)
         else:
-            act = matmul(x, self.w_gate_up, epilogue=ops.EPI_GATED, activation=self.activation, a_rows=sorted_token,
-                         expert_offsets=offsets, n_rows=T * self.top_k, **kb)
+            act = matmul(x, self.w_gate_up, epilogue=ops.EPI_GATED, a_rows=sorted_token,
+                         expert_offsets=offsets, n_rows=T * self.top_k, **self._gated(weights, sorted_pair), **kb)
             debug.region("experts down")
             # each expert's rows go back to the place of their (token, slot) pair
             y = matmul(act, self.w_down, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets, c_rows=sorted_pair, **kb)
@@ -256,7 +277,7 @@ class SparseMoE(FeedForward):
             shared_out.record_stream(main)
             ctx.carry = ops.moe_combine(residual, y, None, weights, self.top_k, shared=shared_out, gate=gate, **then)
         elif self.shared is None:
-            ctx.carry = ops.moe_combine(residual, y, None, weights, self.top_k, **then)
+            ctx.carry = ops.moe_combine(residual, y, None, self._mix(weights), self.top_k, **then)
         else:
             ops.moe_combine(residual, y, None, weights, self.top_k)
             self.shared.forward(x, ctx, residual, row_scale=gate)

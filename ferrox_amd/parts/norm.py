@@ -50,3 +50,29 @@ class RMSNorm(Norm):
 
     def forward(self, h, ctx, rows=None):
         return ops.rmsnorm(h, self.weight, self.eps, ctx.act_dtype, rows=rows)
+
+
+@NORMS.register("layernorm")
+class LayerNorm(Norm):
+    """y = (x - mean) / sqrt(var + eps) * w + b, var the mean of the squared deviations; statistics in float32, read
+    from the float32 residual stream.  It is no RMS norm: `rms_params` declines, so no part fuses it away."""
+    kernel_libraries = ("elementwise",)
+
+    def __init__(self, size: int, eps: float, name: str = "weight", bias_name: str | None = "bias"):
+        """`name`, `bias_name`: what weight and bias are called behind the part's prefix; `bias_name` None: no bias."""
+        self.size, self.eps = int(size), float(eps)
+        self.name, self.bias_name = name, bias_name
+        self.weight = self.bias = None
+
+    def param_specs(self):
+        specs = {self.name: ParamSpec((self.size,), init="ones")}
+        if self.bias_name:
+            specs[self.bias_name] = ParamSpec((self.size,), init="zeros")
+        return specs
+
+    def load(self, fetch):
+        self.weight = fetch(self.name).float().contiguous()
+        self.bias = fetch(self.bias_name).float().contiguous() if self.bias_name else None
+
+    def forward(self, h, ctx, rows=None):
+        return ops.layernorm(h, self.weight, self.bias, self.eps, ctx.act_dtype, rows=rows)

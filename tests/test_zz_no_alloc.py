@@ -59,7 +59,7 @@ def test_decode_attention_that_allocates_nothing(dtype):
         args = (stream, code, p(q), q.stride(0), None, q.stride(0), p(k_pages), p(v_pages), p(table), max_blocks,
                 p(positions), p(items), p(items), n, nh, nkv, hd, bs, window, 1.0 / math.sqrt(hd))
         with_out = lambda out: args[:4] + (p(out),) + args[5:]
-        assert lib.fx_attn_decode(*with_out(want), p(part_o), p(part_ml), splits, chunk, 0, 0, 0, 0, None, None, 0, 0.0, None) == 0, lib.fx_last_error().decode()
+        assert lib.fx_attn_decode(*with_out(want), p(part_o), p(part_ml), splits, chunk, 0, 0, 0, 0, None, None, 0, 0.0, None, 0) == 0, lib.fx_last_error().decode()
         torch.cuda.synchronize()
         # torch's counters see only torch's allocator; the driver's free memory sees a hipMalloc inside the library too
         # (the array's address was looked up by fx_attn_static_init above, so nothing is left to set up)
