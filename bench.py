@@ -405,7 +405,7 @@ def run_workload(name: str, args) -> int:
     return 0
 
 
-# ---- Rafilix, Kovalorn and Fokinex beside the closest existing model, at equal layer sizes ----------------------------------
+# ---- Rafilix, Kovalorn, Fokinex and Panarax beside the closest existing model, at equal layer sizes ----------------------------------
 # Layer sizes that resemble a real model's; every model is four layers of random weights.  The Rafilix layers are
 # measured by kind (all attention, all recurrent) and in the design's usual mixture, the Qwen2-MoE layers have the
 # same width, heads, experts and expert width and no shared expert (Rafilix has none).
@@ -479,7 +479,28 @@ def design_configs(s: dict) -> dict:
         return {"architecture": "Kovalorn", "vocab": s["vocab"], "width": s["width"], "norm": {"eps": 1e-5}, "logit_scale": 1.0,
                 "layers": [{"type": "attention", "mixer": mixer, "mlp": {"kind": "dense", "ff": s["dense_ff"]}}] * 4,
                 "max_positions": 16384}
-    more = {"kovalorn dense": kovalorn_dense(), "fokinex latent": fokinex(["latent"] * 4),
+    # Panarax: gated pre-norm layers (layer norms, an input convolution, gated residuals) around linear attention with
+    # a constant decay, a gated linear recurrent unit, or softmax attention beside a matrix memory; dense feed-forwards
+    # or experts whose weights act on their input.  Beside it (above): Fokinex's attention beside a delta rule and
+    # Kovalorn's attention, both with the same dense feed-forward, and Rafilix's delta-rule layers with experts.
+    def panarax(kinds, sparse=()):
+        dense = {"kind": "dense", "ff": s["dense_ff"]}
+        experts = {"kind": "moe", "expert": {"ff": s["ff"], "limit": 7.0}, "router": {"experts": s["experts"], "top": s["top"]}}
+        H, D = s["heads"], s["dim"]
+        mixers = {
+            "lightning": {"heads": H, "dim": D, "vdim": D, "decay": [1.0 - 0.5 ** (1 + 9 * h / max(1, H - 1)) for h in range(H)]},
+            "rglru": {"width": s["width"] * 5 // 4, "blocks": max(1, s["width"] * 5 // 4 // 256), "conv": 4},
+            "parallel": {"left": {"heads": H, "kv_heads": s["kv_heads"], "dim": D, "vdim": D, "scale": D ** -0.5,
+                                  "q_temp": {"coef": 0.1, "every": 4096}},
+                         "right": {"heads": H, "dim": D, "vdim": D, "gate_cap": 15.0}},
+        }
+        layers = [{"type": kind, "mixer": mixers[kind], "mlp": experts if i in sparse else dense} for i, kind in enumerate(kinds)]
+        return {"architecture": "Panarax", "vocab": s["vocab"], "width": s["width"], "max_positions": 16384, "norm": {"eps": 1e-5},
+                "canon": {"taps": 4}, "layers": layers}
+    more = {"panarax lightning": panarax(["lightning"] * 4), "panarax lru": panarax(["rglru"] * 4),
+            "panarax side by side": panarax(["parallel"] * 4), "panarax experts": panarax(["lightning"] * 4, sparse=(0, 1, 2, 3)),
+            "panarax mixed": panarax(["lightning", "rglru", "parallel", "lightning"], sparse=(1, 3)),
+            "kovalorn dense": kovalorn_dense(), "fokinex latent": fokinex(["latent"] * 4),
             "fokinex side by side": fokinex(["parallel"] * 4),
             "fokinex mixed": fokinex(["latent", "latent", "reader", "parallel"])}
     return {"qwen2-moe": qwen, "rafilix attention": rafilix([attn] * 4), "rafilix recurrent": rafilix([delta] * 4),

@@ -734,7 +734,8 @@ __global__ __launch_bounds__(256) void rglru_gates_kernel(const float* __restric
     const float log_a = -rate * r * softplus_f(load_as_float(lam, lam_dtype, c));
     const float av = expf(log_a);
     a[idx] = av;
-    x[idx] = sqrtf(fmaxf(1.0f - av * av, 0.f)) * i * u[t * ldu + c];
+    // 1 - a^2 = -expm1(2 log a): the difference itself would lose its digits where a is close to one
+    x[idx] = sqrtf(fmaxf(-expm1f(2.0f * log_a), 0.f)) * i * u[t * ldu + c];
 }
 
 FX_API int fx_rglru_gates(void* stream, const float* u, long ldu, const float* logits, const float* bias,

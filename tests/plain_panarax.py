@@ -102,7 +102,9 @@ def softmax_attention(h, w, p, m, eps):
     H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     T = h.shape[0]
     pos = torch.arange(T, dtype=h.dtype)
-    q = (h @ w[p + "q"].T).view(T, H, D) * query_temperature(pos, m["q_temp"]["coef"], m["q_temp"]["every"])[:, None, None]
+    q = (h @ w[p + "q"].T).view(T, H, D)
+    if m.get("q_temp"):
+        q = q * query_temperature(pos, m["q_temp"]["coef"], m["q_temp"]["every"])[:, None, None]
     k = (h @ w[p + "k"].T).view(T, G, D)
     v = unit_rms((h @ w[p + "v"].T).view(T, G, V), eps)
     gate = sigmoid(h @ w[p + "g"].T)                                   # [T, H]
@@ -199,7 +201,7 @@ def mixer(kind, h, w, p, m, eps):
 def layer(x, w, i, entry, cfg, routing=None):
     eps, lp = cfg["norm"]["eps"], f"l{i}."
     h = layer_norm(x, w[lp + "norm1"], w[lp + "norm1.b"], eps)
-    read = h + causal_conv(h, w[lp + "canon1"])
+    read = h + causal_conv(h, w[lp + "canon1"]) if cfg.get("canon") else h
     y = mixer(entry["type"], read, w, lp + "mix.", entry["mixer"], eps)
     x = x + y * sigmoid(h @ w[lp + "rg1"].T + w[lp + "rg1.b"])
     if entry.get("mlp") is None:

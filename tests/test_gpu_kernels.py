@@ -154,9 +154,16 @@ def test_gemm_gate_up(dtype, M, I, K):
     others = {"gelu_tanh": lambda z: 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3))),
               "gelu": lambda z: 0.5 * z * (1.0 + torch.erf(z / math.sqrt(2.0))), "relu": lambda z: z.clamp(min=0.0),
               "silu": plain.silu}
-    assert set(others) == set(ops.ACTIVATIONS)
+    assert set(others) | {"swiglu_clamped"} == set(ops.ACTIVATIONS)
     for name, f in others.items():
         close(ops.gemm(a, w, epilogue=ops.EPI_GATED, activation=name), f(g) * u, dtype, f"{name}(gate)*up")
+    # the clamped gate bounds both factors, and a scale in front of the activation stands for a scaled row of `a`
+    limit, slope = 0.8, 1.702
+    scale = torch.rand(M, generator=torch.Generator().manual_seed(3)).to(DEV) + 0.5
+    gs, us = g * scale.double()[:, None], u * scale.double()[:, None]
+    gc, uc = gs.clamp(max=limit), us.clamp(-limit, limit)
+    close(ops.gemm(a, w, epilogue=ops.EPI_GATED, activation="swiglu_clamped", activation_params=(limit, slope), pre_scale=scale),
+          gc * torch.sigmoid(slope * gc) * (uc + 1.0), dtype, "clamped gate behind a row scale")
     with pytest.raises(ops.KernelError, match="activation"):
         ops.gemm(a, w, epilogue=ops.EPI_GATED, activation="swish2")
 
