@@ -344,9 +344,11 @@ class PagedAttention(Mixer):
                                cache.block_size, self.v_dim)
         return q, rest
 
-    def forward(self, x, ctx, cache, residual, qkv=None, post_norm=None, out_scale: float | None = None) -> None:
+    takes_fresh = True
+
+    def forward(self, x, ctx, cache, residual, qkv=None, post_norm=None, out_scale: float | None = None, fresh: bool = False) -> None:
         """`out_scale`: a constant that the mixer's output is multiplied by on its way into the stream (a mixer that
-        runs beside another one, the two weighted)."""
+        runs beside another one, the two weighted).  `fresh`: `residual` holds nothing yet; the output is stored into it."""
         table = ctx.block_tables[cache.group]
         k_pages, v_pages = cache.pages["k"], cache.pages["v"]
         rot = self.position.rotary()
@@ -428,7 +430,11 @@ class PagedAttention(Mixer):
             ops.attention_decode(q, out, k_pages, v_pages, table, ctx.positions,
                                  items["dec_seq"], items["dec_tok"], *common, max_kv_len=items["max_kv"], **mask)
         debug.region("o_proj")
-        if post_norm is None:
+        if post_norm is None and fresh and (out_scale is None or out_scale == 1.0):
+            self.o_proj(out, epilogue=ops.EPI_STORE_F32, out=residual)
+        elif post_norm is None:
+            if fresh:
+                ops.fill_u32(residual, 0)
             scale = ops.constant_rows(out.device, out_scale, ctx.n_tokens) if out_scale is not None and out_scale != 1.0 else None
             self.o_proj(out, epilogue=ops.EPI_RESID, out=residual, row_scale=scale)
         else:       # the output rows are normed before they join the stream: float32 rows, then one kernel norms and adds

@@ -135,8 +135,9 @@ class GatedPreNormBlock(Block):
         activation).  The last taps - 1 normed rows of every request are part of its state (`block.conv`).
       * a gated residual, G = sigmoid(W x + b) element by element, x being the normed rows the sublayer was handed
         (before the input convolution): a sublayer's float32 output rows pass the gate as they join the stream.
-    A layer without a feed-forward has the first half only.  The sublayers add into a zeroed float32 buffer in
-    place of the stream (their last product's epilogue), which one kernel then gates and adds."""
+    A layer without a feed-forward has the first half only.  A sublayer leaves its output in a float32 buffer in
+    place of the stream (stored by its last product if it says `takes_fresh`, else added into a zeroed buffer),
+    which one kernel then gates and adds."""
     slots = {"norm1": NORMS, "mixer": MIXERS, "norm2": NORMS, "ffn": FEED_FORWARDS}
     optional_slots = ("norm2", "ffn")
     kernel_libraries = ("elementwise", "gemm", "recurrent")
@@ -181,6 +182,17 @@ class GatedPreNormBlock(Block):
     def state_shapes(self) -> dict:
         return {"conv": ((self.hidden_size, self.conv_taps - 1), torch.float32)} if self.conv_taps else {}
 
+    @staticmethod
+    def _into(part, out, x, ctx, *cache):
+        """The sublayer's output rows in `out`: a part that says `takes_fresh` stores them with its last product,
+        any other adds them into a zeroed buffer."""
+        from .. import ops
+        if getattr(part, "takes_fresh", False):
+            part.forward(x, ctx, *cache, out, fresh=True)
+        else:
+            ops.fill_u32(out, 0)
+            part.forward(x, ctx, *cache, out)
+
     def _join(self, h, out, gate, x):
         from .. import ops
         debug.region("residual gate")
@@ -200,13 +212,11 @@ class GatedPreNormBlock(Block):
             read = ops.short_conv(x, self.taps, cache.state["block.conv"], ctx.token_seq, sequence_starts(ctx), ctx.slot_ids,
                                   ctx.n_seqs, activation=None, add_input=True, out_dtype=x.dtype)
         out = torch.empty_like(h)
-        ops.fill_u32(out, 0)
-        self.mixer.forward(read, ctx, cache, out)
+        self._into(self.mixer, out, read, ctx, cache)
         self._join(h, out, self.gate1, x)
         if self.ffn is None:
             return
         debug.region("norm")
         x = self.norm2.forward(h, ctx)
-        ops.fill_u32(out, 0)
-        self.ffn.forward(x, ctx, out)
+        self._into(self.ffn, out, x, ctx)
         self._join(h, out, self.gate2, x)

@@ -80,7 +80,10 @@ class SideBySide(Mixer):
             if rms is None:
                 raise ValueError(f"member '{name}': its output's norm must be an RMS norm with a weight")
             rows = torch.empty_like(residual)
-            ops.fill_u32(rows, 0)
-            m.forward(x, ctx, own, rows)
+            if getattr(m, "takes_fresh", False):      # the member stores its rows; any other adds into zeroed ones
+                m.forward(x, ctx, own, rows, fresh=True)
+            else:
+                ops.fill_u32(rows, 0)
+                m.forward(x, ctx, own, rows)
             debug.region("member norm")
             ops.rmsnorm_add(residual, rows, rms[0], rms[1])

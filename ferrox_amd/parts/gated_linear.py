@@ -37,8 +37,15 @@ def longest_portion(ctx) -> int:
     return max((ctx.q_starts[s + 1] - ctx.q_starts[s] for s in range(ctx.n_seqs)), default=0)
 
 
-def _add_out(o_proj, y, ctx, residual, out_scale):
+def _add_out(o_proj, y, ctx, residual, out_scale, fresh=False):
+    """The output projection into `residual`: added, or, where the caller says that `residual` holds nothing yet
+    (`fresh`), stored."""
     debug.region("o_proj")
+    if fresh and (out_scale is None or out_scale == 1.0):
+        o_proj(y, epilogue=ops.EPI_STORE_F32, out=residual)
+        return
+    if fresh:
+        ops.fill_u32(residual, 0)
     scale = ops.constant_rows(y.device, out_scale, ctx.n_tokens) if out_scale is not None and out_scale != 1.0 else None
     o_proj(y, epilogue=ops.EPI_RESID, out=residual, row_scale=scale)
 
@@ -83,7 +90,9 @@ class DecayAttention(Mixer):
     def state_shapes(self) -> dict:
         return {"S": ((self.n_heads, self.v_dim, self.key_dim), torch.float32)}      # transposed: [head][value][key]
 
-    def forward(self, x, ctx, cache, residual, out_scale: float | None = None) -> None:
+    takes_fresh = True       # forward(..., fresh=True): `residual` holds nothing yet, the output is stored into it
+
+    def forward(self, x, ctx, cache, residual, out_scale: float | None = None, fresh: bool = False) -> None:
         H, D, V, QK = self.n_heads, self.key_dim, self.v_dim, self.qk_width
         debug.region("linear in")
         # the activation is applied to the float32 sums as they are stored: what the recurrence reads is float32
@@ -94,7 +103,7 @@ class DecayAttention(Mixer):
                             sequence_starts(ctx), ctx.slot_ids, ctx.n_seqs, H, H, D, V)
         debug.region("linear out")
         y = ops.gated_head_norm(o, gate, self.norm_w, self.norm_eps, 1, H * V, ctx.act_dtype)      # all heads as one row
-        _add_out(self.o_proj, y, ctx, residual, out_scale)
+        _add_out(self.o_proj, y, ctx, residual, out_scale, fresh)
 
 
 @MIXERS.register("matrix_memory")
@@ -140,7 +149,9 @@ class MatrixMemory(Mixer):
         return {"S": ((self.n_heads, self.v_dim + 1, self.key_dim), torch.float32),      # transposed; the last column is n
                 "m": ((self.n_heads,), torch.float32)}
 
-    def forward(self, x, ctx, cache, residual, out_scale: float | None = None) -> None:
+    takes_fresh = True
+
+    def forward(self, x, ctx, cache, residual, out_scale: float | None = None, fresh: bool = False) -> None:
         H, D, V, QK, VW = self.n_heads, self.key_dim, self.v_dim, self.qk_width, self.v_width
         debug.region("memory in")
         proj = self.w_in(x, epilogue=ops.EPI_STORE_F32)
@@ -155,7 +166,7 @@ class MatrixMemory(Mixer):
                                 ctx.slot_ids, ctx.n_seqs, H, H, D, V, q_scale=D ** -0.5, normalizer=True)
         debug.region("memory out")
         y = ops.gated_head_norm(o, proj[:, g0:i0], self.norm_w, self.norm_eps, H, V, ctx.act_dtype, denominators=(nq, m))
-        _add_out(self.o_proj, y, ctx, residual, out_scale)
+        _add_out(self.o_proj, y, ctx, residual, out_scale, fresh)
 
 
 @MIXERS.register("rglru")
@@ -201,7 +212,9 @@ class RGLRU(Mixer):
     def state_shapes(self) -> dict:
         return {"S": ((self.width,), torch.float32), "conv": ((self.width, self.conv_taps - 1), torch.float32)}
 
-    def forward(self, x, ctx, cache, residual, out_scale: float | None = None) -> None:
+    takes_fresh = True
+
+    def forward(self, x, ctx, cache, residual, out_scale: float | None = None, fresh: bool = False) -> None:
         C, B, T = self.width, self.n_blocks, ctx.n_tokens
         cb = C // B
         debug.region("lru in")
@@ -220,4 +233,4 @@ class RGLRU(Mixer):
         # (the gates' biases join inside: the grouped product has one bias for all groups)
         y = ops.rglru(u, logits, self.gate_bias, B, self.lam, proj[:, :C], cache.state["S"], starts, ctx.slot_ids, ctx.n_seqs,
                       longest_portion(ctx), ctx.act_dtype, rate=self.RATE)
-        _add_out(self.o_proj, y, ctx, residual, out_scale)
+        _add_out(self.o_proj, y, ctx, residual, out_scale, fresh)

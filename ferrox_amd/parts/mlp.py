@@ -37,10 +37,17 @@ class GatedMLP(FeedForward):
         """The feed-forward's output as float32 [T, H], added to nothing."""
         return self.down(self.gate_up(x, epilogue=ops.EPI_GATED, activation=self.activation), epilogue=ops.EPI_STORE_F32)
 
-    def forward(self, x, ctx, residual, row_scale=None) -> None:
+    takes_fresh = True       # forward(..., fresh=True): `residual` holds nothing yet, the output is stored into it
+
+    def forward(self, x, ctx, residual, row_scale=None, fresh: bool = False) -> None:
         debug.region("mlp gate/up")
         act = self.gate_up(x, epilogue=ops.EPI_GATED, activation=self.activation)
         debug.region("mlp down")
+        if fresh and row_scale is None:
+            self.down(act, epilogue=ops.EPI_STORE_F32, out=residual)
+            return
+        if fresh:
+            ops.fill_u32(residual, 0)
         self.down(act, epilogue=ops.EPI_RESID, out=residual, row_scale=row_scale)
 
 

@@ -80,8 +80,9 @@ def test_stop_ids_are_one_or_several():
 
 
 def test_registry_is_closed(tmp_path):
-    assert known_architectures() == ["Fokinex", "Kovalorn", "Qwen2MoeForCausalLM", "Rafilix"]
+    assert known_architectures() == ["Fokinex", "Kovalorn", "Panarax", "Qwen2MoeForCausalLM", "Rafilix"]
     assert resolve({"architecture": "Fokinex"}).model_type == "fokinex"
+    assert resolve({"architecture": "Panarax"}).model_type == "panarax"
     assert resolve({"architecture": "Rafilix"}).model_type == "rafilix"
     assert resolve({"architecture": "Kovalorn"}).model_type == "kovalorn"
     with pytest.raises(ConfigError) as e:
