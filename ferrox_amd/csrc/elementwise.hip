@@ -60,6 +60,33 @@ __global__ __launch_bounds__(256) void layernorm_kernel(const float* __restrict_
     __shared__ float red[4];
     const int r = blockIdx.x;
     const float* x = h + (size_t)(rows ? rows[r] : r) * ld;
+    if (H <= 256 * 16) {   // the row stays in registers: one pass over memory, weight and bias fetched meanwhile
+        float xv[16], wv[16], bv[16];
+        float sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int c = threadIdx.x + i * 256;
+            xv[i] = c < H ? x[c] : 0.f;
+            sum += xv[i];
+        }
+        load_strided_as_float<16, 256>(w, w_dtype, threadIdx.x, H, wv);
+        if (b) load_strided_as_float<16, 256>(b, w_dtype, threadIdx.x, H, bv);
+        const float mean = block_sum<4>(sum, red) / (float)H;
+        __syncthreads();                               // (`red` is used again)
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const float d = threadIdx.x + i * 256 < H ? xv[i] - mean : 0.f;
+            ss = fmaf(d, d, ss);
+        }
+        const float rstd = 1.0f / sqrtf(block_sum<4>(ss, red) / (float)H + eps);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int c = threadIdx.x + i * 256;
+            if (c < H) from_float(out + (size_t)r * H + c, (xv[i] - mean) * rstd * wv[i] + (b ? bv[i] : 0.f));
+        }
+        return;
+    }
     float sum = 0.f;
     for (int c = threadIdx.x; c < H; c += 256) sum += x[c];
     const float mean = block_sum<4>(sum, red) / (float)H;

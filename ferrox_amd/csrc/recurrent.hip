@@ -239,6 +239,35 @@ FX_API int fx_small_rows_pair(void* stream, const float* x0, long ldx0, const fl
 }
 
 // ---------------------------------------------------------------------------
+// A block-diagonal float32 product of few rows in one launch: the K-wide part j of row t, times the transposed matrix
+// wt[j] [K, N] of that part, out[t, j, n] = sum_k x[t, j K + k] * wt[j, k, n], k ascending in one accumulator.  These
+// are the gates of a recurrent unit whose channels are cut into parts with a square matrix each; a decode step's few
+// rows would wait in a tiled product's launch for nothing.  Grid: (ceil(N / 256), rows, parts).
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void small_rows_parts_kernel(const float* __restrict__ x, long ldx, const float* __restrict__ wt,
+                                                               float* __restrict__ out, int K, int N, int parts) {
+    __shared__ float xs[PAIR_MAX_K];
+    const int t = blockIdx.y, j = blockIdx.z, n = blockIdx.x * 256 + threadIdx.x;
+    for (int k = threadIdx.x; k < K; k += 256) xs[k] = x[(size_t)t * ldx + (size_t)j * K + k];
+    __syncthreads();
+    if (n >= N) return;
+    const float* w = wt + (size_t)j * K * N;
+    float acc = 0.f;
+#pragma unroll 8
+    for (int k = 0; k < K; ++k) acc = fmaf(xs[k], w[(size_t)k * N + n], acc);
+    out[((size_t)t * parts + j) * N + n] = acc;
+}
+
+FX_API int fx_small_rows_parts(void* stream, const float* x, long ldx, const float* wt, float* out, int K, int N, int parts, int T) {
+    FX_REQUIRE(T >= 0 && T <= 65535 && parts >= 1 && parts <= 65535, "small_rows_parts: %d rows of %d parts", T, parts);
+    FX_REQUIRE(K >= 1 && K <= PAIR_MAX_K && N >= 1 && ldx >= (long)parts * K, "small_rows_parts: parts of %d columns (up to %d) in rows of %ld", K, PAIR_MAX_K, ldx);
+    if (T == 0) return 0;
+    small_rows_parts_kernel<<<dim3((N + 255) / 256, T, parts), 256, 0, (hipStream_t)stream>>>(x, ldx, wt, out, K, N, parts);
+    FX_CHECK_LAUNCH("small_rows_parts");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
 // The recurrence.  Per head, with S [D, V] carried from token to token:
 //   S <- diag(decay_t) S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T;  o_t = S^T q_t
 // Tokens follow each other; columns of S never meet.  A wave owns 64 / LPC columns, LPC = 16 or 32 lanes to a
@@ -462,6 +491,32 @@ __global__ __launch_bounds__(256) void gated_head_norm_kernel(const float* __res
     }
 }
 
+// The same for long rows (all heads normed as one row of thousands of channels): a block per (token, head), so that a
+// decode step's few rows are not one wave's long loop each.
+template <typename T>
+__global__ __launch_bounds__(256) void gated_row_norm_kernel(const float* __restrict__ o, long ldo, const float* __restrict__ gate,
+                                                             long ldg, const void* __restrict__ w, int w_dtype, int w_stride, T* __restrict__ y,
+                                                             long ldy, int H, int V, float eps, int gate_act,
+                                                             const float* __restrict__ nq, const float* __restrict__ m) {
+    __shared__ float red[4];
+    const int row = blockIdx.x, t = row / H, h = row - t * H;
+    const float* src = o + (size_t)t * ldo + (size_t)h * V;
+    float inv_den = 1.0f;
+    if (nq) inv_den = 1.0f / (fmaxf(fabsf(nq[row]), expf(-m[row])) + 1e-6f);
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < V; i += 256) {
+        const float x = src[i] * inv_den;
+        ss = fmaf(x, x, ss);
+    }
+    ss = block_sum<4>(ss, red);
+    const float scale = 1.0f / sqrtf(ss / (float)V + eps);
+    for (int i = threadIdx.x; i < V; i += 256) {
+        const float gx = gate[(size_t)t * ldg + (size_t)h * V + i];
+        const float gt = (gate_act ? gx : 1.0f) / (1.0f + expf(-gx));
+        from_float(y + (size_t)t * ldy + (size_t)h * V + i, src[i] * inv_den * scale * load_as_float(w, w_dtype, (size_t)h * w_stride + i) * gt);
+    }
+}
+
 FX_API int fx_gated_head_norm(void* stream, int out_dtype, const float* o, long ldo, const float* gate, long ldg,
                               const void* w, int w_dtype, int w_per_head, void* y, long ldy, int T, int H, int V, float eps,
                               int gate_act, const float* nq, const float* m) {
@@ -473,6 +528,12 @@ FX_API int fx_gated_head_norm(void* stream, int out_dtype, const float* o, long 
     if (T == 0) return 0;
     const int rows = T * H, ws = w_per_head ? V : 0;
     hipStream_t s = (hipStream_t)stream;
+    if (V > 512 && (out_dtype == FX_F32 || out_dtype == FX_BF16)) {
+        if (out_dtype == FX_F32) gated_row_norm_kernel<float><<<rows, 256, 0, s>>>(o, ldo, gate, ldg, w, w_dtype, ws, (float*)y, ldy, H, V, eps, gate_act, nq, m);
+        else gated_row_norm_kernel<bf16><<<rows, 256, 0, s>>>(o, ldo, gate, ldg, w, w_dtype, ws, (bf16*)y, ldy, H, V, eps, gate_act, nq, m);
+        FX_CHECK_LAUNCH("gated_head_norm");
+        return 0;
+    }
     if (out_dtype == FX_F32)
         gated_head_norm_kernel<float><<<(rows + 3) / 4, 256, 0, s>>>(o, ldo, gate, ldg, w, w_dtype, ws, (float*)y, ldy, rows, H, V, eps, gate_act, nq, m);
     else if (out_dtype == FX_BF16)
@@ -764,13 +825,23 @@ __global__ __launch_bounds__(NW * 64) void rglru_scan_kernel(const float* __rest
     const int n = t1 - t0, per = (n + NW - 1) / NW;
     const int w0 = min(t0 + wave * per, t1), w1 = min(w0 + per, t1);
     const bool in = c < C;
+    constexpr int P = 8;                             // tokens whose operands are asked for together
     float A = 1.f, B = 0.f;
     if (NW > 1) {
         if (in)
-            for (int t = w0; t < w1; ++t) {
-                const float av = a[(size_t)t * C + c];
-                B = fmaf(av, B, x[(size_t)t * C + c]);
-                A *= av;
+            for (int t = w0; t < w1; t += P) {
+                float av[P], xv[P];
+#pragma unroll
+                for (int p = 0; p < P; ++p) {            // (past the stretch: the map that changes nothing)
+                    const bool live = t + p < w1;
+                    av[p] = live ? a[(size_t)(t + p) * C + c] : 1.f;
+                    xv[p] = live ? x[(size_t)(t + p) * C + c] : 0.f;
+                }
+#pragma unroll
+                for (int p = 0; p < P; ++p) {
+                    B = fmaf(av[p], B, xv[p]);
+                    A *= av[p];
+                }
             }
         A_of[wave][lane] = A;
         B_of[wave][lane] = B;
@@ -779,10 +850,20 @@ __global__ __launch_bounds__(NW * 64) void rglru_scan_kernel(const float* __rest
     float S = in ? state[(size_t)slots[s] * C + c] : 0.f;
     for (int w = 0; w < wave; ++w) S = fmaf(A_of[w][lane], S, B_of[w][lane]);
     if (!in) return;
-#pragma unroll 4
-    for (int t = w0; t < w1; ++t) {
-        S = fmaf(a[(size_t)t * C + c], S, x[(size_t)t * C + c]);
-        from_float(y + (size_t)t * ldy + c, S * gelu_tanh_f(b[(size_t)t * ldb + c]));
+    for (int t = w0; t < w1; t += P) {
+        float av[P], xv[P], bv[P];
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const bool live = t + p < w1;
+            av[p] = live ? a[(size_t)(t + p) * C + c] : 1.f;
+            xv[p] = live ? x[(size_t)(t + p) * C + c] : 0.f;
+            bv[p] = live ? b[(size_t)(t + p) * ldb + c] : 0.f;
+        }
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            S = fmaf(av[p], S, xv[p]);
+            if (t + p < w1) from_float(y + (size_t)(t + p) * ldy + c, S * gelu_tanh_f(bv[p]));
+        }
     }
     if (wave == NW - 1) state[(size_t)slots[s] * C + c] = S;
 }

@@ -98,6 +98,7 @@ _sigs = {
                                         c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int],
     ("recurrent", "fx_small_rows_pair"): [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_int,
                                           c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_int, c_int],
+    ("recurrent", "fx_small_rows_parts"): [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int],
     ("recurrent", "fx_gated_head_norm"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_int, c_void_p,
                                           c_long, c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p],
     ("elementwise", "fx_head_norm_kv_write"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int,
@@ -1112,6 +1113,20 @@ def gated_head_norm(o, gate, weight, eps: float, n_heads: int, v_dim: int, out_d
           _p(weight), dtype_code(weight.dtype), 1 if (weight.numel() == H * V and H > 1) else 0, _p(y), y.stride(0), T, H, V,
           float(eps), HEAD_GATES[gate_activation], _p(nq), _p(m))
     return y
+
+
+def small_rows_parts(x, wt):
+    """A block-diagonal float32 product of few rows, one launch: x float32 rows [T, parts * K] (any row stride), wt
+    contiguous float32 [parts, K, N] (every part's matrix transposed); returns contiguous [T, parts, N] with
+    out[t, j] = x[t, j K:(j + 1) K] @ wt[j], the sums over k ascending in one accumulator, as `gemm` does in float32."""
+    T = x.shape[0]
+    if wt.dtype != torch.float32 or wt.dim() != 3 or not wt.is_contiguous() or wt.shape[1] > SMALL_ROWS_MAX_K:
+        raise KernelError(f"small_rows_parts: transposed weights {tuple(wt.shape)} ({wt.dtype})")
+    parts, K, N = wt.shape
+    _f32_rows(x, "small_rows_parts: x", parts * K)
+    out = torch.empty((T, parts, N), dtype=torch.float32, device=x.device)
+    _call("recurrent", "fx_small_rows_parts", _stream(), _p(x), x.stride(0), _p(wt), _p(out), K, N, parts, T)
+    return out
 
 
 def gated_outer(q, k, v, keep, take, state, seq_starts, slot_ids, n_seqs: int, n_heads: int, n_kv_heads: int, key_dim: int,

@@ -184,7 +184,7 @@ class RGLRU(Mixer):
         if not 1 <= self.conv_taps <= 16:
             raise ValueError(f"conv_taps {conv_taps}: the convolution kernel takes 1..16 taps")
         self.names = dict(self.TENSORS, **(names or {}))
-        self.w_in = self.taps = self.conv_bias = self.w_gates = self.gate_bias = self.lam = self.o_proj = None
+        self.w_in = self.taps = self.conv_bias = self.w_gates = self.w_gates_t = self.gate_bias = self.lam = self.o_proj = None
 
     def param_specs(self):
         W, C, B, n = self.hidden_size, self.width, self.n_blocks, self.names
@@ -206,6 +206,8 @@ class RGLRU(Mixer):
         # per part j one matrix [2 cb, cb]: the recurrence gate's rows, then the input gate's
         self.w_gates = torch.cat([fetch(n["rec_gate"]).float(), fetch(n["in_gate"]).float()], dim=1).contiguous()
         self.gate_bias = torch.cat([fetch(n["rec_gate_bias"]).float(), fetch(n["in_gate_bias"]).float()], dim=1).contiguous()
+        # (a transposed copy for the few rows of a decode step, where the parts' products are one small launch)
+        self.w_gates_t = self.w_gates.transpose(1, 2).contiguous()
         self.lam = fetch(n["lam"]).float().contiguous()
         self.o_proj = Linear(fetch(n["o"]))
 
@@ -225,10 +227,13 @@ class RGLRU(Mixer):
                            activation=None, bias=self.conv_bias)
         debug.region("lru gates")
         # the gates' products, a part of the channels each: part j of token t is row t*B + j of [T*B, cb]
-        rows, offsets = head_groups(u.device, T, B)
-        logits = torch.empty((T * B, 2 * cb), dtype=torch.float32, device=u.device)
-        ops.gemm(u.view(T * B, cb), self.w_gates, a_rows=rows, c_rows=rows, expert_offsets=offsets, n_rows=T * B,
-                 epilogue=ops.EPI_STORE_F32, out=logits)
+        if T <= ops.SMALL_ROWS_MAX and cb <= ops.SMALL_ROWS_MAX_K:
+            logits = ops.small_rows_parts(u, self.w_gates_t)
+        else:
+            rows, offsets = head_groups(u.device, T, B)
+            logits = torch.empty((T * B, 2 * cb), dtype=torch.float32, device=u.device)
+            ops.gemm(u.view(T * B, cb), self.w_gates, a_rows=rows, c_rows=rows, expert_offsets=offsets, n_rows=T * B,
+                     epilogue=ops.EPI_STORE_F32, out=logits)
         debug.region("linear recurrence")
         # (the gates' biases join inside: the grouped product has one bias for all groups)
         y = ops.rglru(u, logits, self.gate_bias, B, self.lam, proj[:, :C], cache.state["S"], starts, ctx.slot_ids, ctx.n_seqs,

@@ -216,6 +216,42 @@ def test_gated_linear_recurrent_unit(C, parts, lengths):
         t0 += n
 
 
+@pytest.mark.parametrize("H, V, per_head, den", [(3, 20, True, True), (1, 1500, False, False), (2, 640, True, True), (4, 64, False, False)])
+def test_read_out_norm_with_weights_per_head_and_denominators(H, V, per_head, den):
+    """Short rows (a wave each) and long ones (a block each), a weight per head and channel, the memory's denominators."""
+    from ferrox_amd import ops
+    gen = torch.Generator().manual_seed(V)
+    T = 5
+    o, gate = torch.randn(T, H * V, generator=gen), torch.randn(T, H * V, generator=gen)
+    w = torch.randn(H * V if per_head else V, generator=gen)
+    nq, m = torch.randn(T, H, generator=gen) * 2, torch.randn(T, H, generator=gen)
+    y = ops.gated_head_norm(o.cuda(), gate.cuda(), w.cuda(), 1e-5, H, V, torch.float32,
+                            denominators=(nq.cuda(), m.cuda()) if den else None)
+    x = o.to(F64).view(T, H, V)
+    if den:
+        x = x / (torch.maximum(nq.to(F64).abs(), torch.exp(-m.to(F64))) + 1e-6)[:, :, None]
+    want = plain.unit_rms(x, 1e-5) * (w.to(F64).view(H, V) if per_head else w.to(F64)) * plain.sigmoid(gate.to(F64).view(T, H, V))
+    assert torch.allclose(y.cpu().to(F64), want.reshape(T, H * V), rtol=2e-5, atol=2e-5)
+
+
+def test_block_diagonal_product_for_few_rows():
+    """The small launch of a decode step gives what the grouped product gives for many rows."""
+    from ferrox_amd import ops
+    from ferrox_amd.parts.latent import head_groups
+    gen = torch.Generator().manual_seed(4)
+    for T, parts, K, N in ((1, 3, 16, 32), (7, 5, 80, 160), (32, 2, 300, 70)):
+        x = torch.randn(T, parts * K + 3, generator=gen).cuda()[:, :parts * K]
+        w = torch.randn(parts, N, K, generator=gen).cuda()
+        got = ops.small_rows_parts(x, w.transpose(1, 2).contiguous())
+        want = torch.einsum("tjk,jnk->tjn", x.cpu().to(F64).view(T, parts, K), w.cpu().to(F64))
+        assert torch.allclose(got.cpu().to(F64), want, rtol=1e-5, atol=1e-4)
+        rows, offsets = head_groups("cuda:0", T, parts)
+        tiled = torch.empty(T * parts, N, device="cuda")
+        ops.gemm(x.contiguous().view(T * parts, K), w, a_rows=rows, c_rows=rows, expert_offsets=offsets, n_rows=T * parts,
+                 epilogue=ops.EPI_STORE_F32, out=tiled)
+        assert torch.equal(got.view(T * parts, N), tiled), "few rows and many rows round differently"
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_layer_norm_gated_add_and_position_table(dtype):
     from ferrox_amd import ops
@@ -227,6 +263,10 @@ def test_layer_norm_gated_add_and_position_table(dtype):
     tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
     assert torch.allclose(ops.layernorm(h, w, b, 1e-5, dtype).cpu().to(F64), want, **tol)
     assert torch.allclose(ops.layernorm(h, w, b, 1e-5, dtype, rows=rows).cpu().to(F64), want[[5, 0, 5]], **tol)
+    wide = (torch.randn(3, 4500, generator=gen) * 2 - 1).cuda()        # (rows beyond what a block keeps in registers)
+    ww, wb = torch.randn(4500, generator=gen).cuda(), torch.randn(4500, generator=gen).cuda()
+    assert torch.allclose(ops.layernorm(wide, ww, wb, 1e-6, dtype).cpu().to(F64),
+                          plain.layer_norm(wide.cpu().to(F64), ww.cpu().to(F64), wb.cpu().to(F64), 1e-6), **tol)
     y, g = torch.randn(7, 70, generator=gen).cuda(), torch.randn(7, 70, generator=gen).cuda() * 3
     out = h.clone()
     ops.gated_add(out, y, g)
