@@ -5,6 +5,9 @@
     python bench.py --workload config3|config4|config5           serving runs through Engine.generate
     python bench.py --kernel-table decode_b1|decode_b8|decode_b16|..|decode_b64|prefill_128|prefill_512|prefill_2048|prefill_4096 [--out FILE]
                                                                  per-kernel times under rocprofv3 (a child process)
+    python bench.py --compare-designs [--design TEXT] [--design-size 1k|2k]
+                                                                 four layers of each other design (Rafilix, Kovalorn, Fokinex, Panarax)
+                                                                 beside the closest models at equal sizes: prefill and decode
 
 Model: the layer sizes of Qwen1.5-MoE-A2.7B with seeded random bf16 weights
 N(0, 0.02) made on the GPU, seeded random token ids.  A "step" is one decode
@@ -800,8 +803,8 @@ def main() -> int:
                     help="per-kernel times of one workload, measured by rocprofv3 around a child process")
     ap.add_argument("--out", help="with --kernel-table: also write the table to this file")
     ap.add_argument("--compare-designs", action="store_true",
-                    help="Rafilix layers (all attention, all recurrent, mixed) and Kovalorn layers (with keys of their own, "
-                         "reading another layer's) beside Qwen2-MoE layers of equal sizes: "
+                    help="Rafilix layers (all attention, all recurrent, mixed), Kovalorn layers (with keys of their own, "
+                         "reading another layer's), Fokinex and Panarax layers (by mixer, and mixed) beside Qwen2-MoE layers of equal sizes: "
                          "prefill of --ctx tokens, decode at batch 1 and --batch; random weights, four layers each")
     ap.add_argument("--design-size", choices=sorted(DESIGN_SIZES), help="with --compare-designs: one size only")
     ap.add_argument("--design", help="with --compare-designs: only the designs whose name holds this text")

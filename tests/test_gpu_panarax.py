@@ -557,3 +557,33 @@ def test_command_line_and_replay(tmp_path_factory):
     for step, want_rows in ((0, [la[0], la[16]]), (1, [lb[2]]), (2, [lb[3], la[29]])):
         got = torch.from_numpy(np.fromfile(os.path.join(out_dir, f"{step}.f32"), dtype="<f4").reshape(-1, V))
         assert float(u.row_errors(got, torch.stack(want_rows)).max()) <= u.LIMIT["float32"], step
+
+
+def test_replay_of_a_model_that_keeps_no_pages(tmp_path_factory):
+    """Layers of recurrent mixers alone: the cache manager has no group of pages, requests hold state slots only."""
+    import json
+    import os
+    import subprocess
+    import sys
+
+    import numpy as np
+    from conftest import ROOT
+    cfg = u.config([u.rglru_layer(mlp=u.moe(4, 2, 16, 1.0)), u.lightning_layer(mlp=u.dense(24))], taps=2)
+    weights = u.make_weights(cfg, 5)
+    folder = u.write_model(str(tmp_path_factory.mktemp("panarax_no_pages")), cfg, weights)
+    a, b = u.random_tokens(cfg["vocab"], 70, 1), u.random_tokens(cfg["vocab"], 9, 2)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:65], "want": [64]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[65:66], "want": [0]}, {"id": "b", "tokens": b[:8], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "b", "tokens": b[8:], "want": [0]}, {"id": "a", "tokens": a[66:], "want": [3]}], "end": ["a", "b"]},
+             {"step": 3, "entries": [{"id": "c", "tokens": b, "want": [8]}], "end": ["c"]}]       # the slot that b left
+    out_dir = str(tmp_path_factory.mktemp("panarax_no_pages_out"))
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", "float32",
+                          "--out", out_dir, "--max-tokens", "192", "--max-seqs", "2"], input="\n".join(json.dumps(s) for s in steps) + "\n",
+                         capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr[-2000:]
+    w = u.as_float64(weights)
+    la, lb = plain.forward(cfg, w, a), plain.forward(cfg, w, b)
+    V = cfg["vocab"]
+    for step, want_rows in ((0, [la[64]]), (1, [la[65]]), (2, [lb[8], la[69]]), (3, [lb[8]])):
+        got = torch.from_numpy(np.fromfile(os.path.join(out_dir, f"{step}.f32"), dtype="<f4").reshape(-1, V))
+        assert float(u.row_errors(got, torch.stack(want_rows)).max()) <= u.LIMIT["float32"], step
