@@ -618,6 +618,60 @@ FX_API int fx_temp_unit_kv_write(void* stream, int dtype, const float* qkv, long
 }
 
 // ---------------------------------------------------------------------------
+// The gated add and the layer norm that follows it, one launch: h += y * sigmoid(g), then
+// out = (h - mean) / sqrt(var + eps) * w + b of the new row.  Rows of up to 4,096 columns stay in registers; the
+// sums are those of the two kernels it stands for (the same order, so the same bits).  One block per row.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void gated_add_layernorm_kernel(float* __restrict__ h, const float* __restrict__ y,
+                                                                  const float* __restrict__ g, const void* __restrict__ w,
+                                                                  const void* __restrict__ b, int w_dtype, T* __restrict__ out,
+                                                                  int H, float eps) {
+    __shared__ float red[4];
+    const size_t row = (size_t)blockIdx.x * H;
+    float xv[16], wv[16], bv[16];
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int c = threadIdx.x + i * 256;
+        xv[i] = 0.f;
+        if (c < H) {
+            xv[i] = h[row + c] + y[row + c] / (1.0f + expf(-g[row + c]));
+            h[row + c] = xv[i];
+        }
+        sum += xv[i];
+    }
+    load_strided_as_float<16, 256>(w, w_dtype, threadIdx.x, H, wv);
+    if (b) load_strided_as_float<16, 256>(b, w_dtype, threadIdx.x, H, bv);
+    const float mean = block_sum<4>(sum, red) / (float)H;
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const float d = threadIdx.x + i * 256 < H ? xv[i] - mean : 0.f;
+        ss = fmaf(d, d, ss);
+    }
+    const float rstd = 1.0f / sqrtf(block_sum<4>(ss, red) / (float)H + eps);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int c = threadIdx.x + i * 256;
+        if (c < H) from_float(out + row + c, (xv[i] - mean) * rstd * wv[i] + (b ? bv[i] : 0.f));
+    }
+}
+
+FX_API int fx_gated_add_layernorm(void* stream, int out_dtype, float* h, const float* y, const float* g, const void* w,
+                                  const void* b, int w_dtype, void* out, int T, int H, float eps) {
+    FX_REQUIRE(T >= 0 && H > 0 && H <= 4096 && w, "gated_add_layernorm: %d rows of %d columns (up to 4096)", T, H);
+    FX_REQUIRE(w_dtype == FX_F32 || w_dtype == FX_BF16, "gated_add_layernorm: unknown weight dtype %d", w_dtype);
+    if (T == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (out_dtype == FX_F32) gated_add_layernorm_kernel<float><<<T, 256, 0, s>>>(h, y, g, w, b, w_dtype, (float*)out, H, eps);
+    else if (out_dtype == FX_BF16) gated_add_layernorm_kernel<bf16><<<T, 256, 0, s>>>(h, y, g, w, b, w_dtype, (bf16*)out, H, eps);
+    else return fx_fail("gated_add_layernorm: unknown output dtype %d", out_dtype);
+    FX_CHECK_LAUNCH("gated_add_layernorm");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
 // Latent attention, what a layer keeps per position.  `down` [T, R + rd] float32 is the down-projection of a
 // token: R latent channels, then a key part of rd dimensions that all heads share.  One block per token:
 //   c = down[:R] / sqrt(mean(down[:R]^2) + eps) * w          (statistics and product in float32)

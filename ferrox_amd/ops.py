@@ -62,6 +62,8 @@ _sigs = {
     ("elementwise", "fx_embed"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_int],
     ("elementwise", "fx_layernorm"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_long],
     ("elementwise", "fx_gated_add"): [c_void_p, c_void_p, c_void_p, c_void_p, c_long],
+    ("elementwise", "fx_gated_add_layernorm"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                                                c_int, c_int, c_float],
     ("elementwise", "fx_temp_unit_kv_write"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p,
                                                c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                                c_float, c_int, c_int, c_float],
@@ -207,6 +209,26 @@ def gated_add(h: torch.Tensor, y: torch.Tensor, gate_logits: torch.Tensor) -> No
         if t.dtype != torch.float32 or not t.is_contiguous() or t.shape != h.shape:
             raise KernelError("gated_add wants contiguous float32 tensors of one shape")
     _call("elementwise", "fx_gated_add", _stream(), _p(h), _p(y), _p(gate_logits), h.numel())
+
+
+GATED_ADD_NORM_MAX = 4096       # the widest row that the gated add keeps in registers for the norm behind it
+
+
+def gated_add_layernorm(h: torch.Tensor, y: torch.Tensor, gate_logits: torch.Tensor, weight: torch.Tensor,
+                        bias: torch.Tensor | None, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """`gated_add(h, y, gate_logits)` and `layernorm(h, weight, bias, eps, out_dtype)` of the new rows in one launch
+    (rows of up to GATED_ADD_NORM_MAX columns); returns the normed rows."""
+    for t in (h, y, gate_logits):
+        if t.dtype != torch.float32 or not t.is_contiguous() or t.shape != h.shape or t.dim() != 2:
+            raise KernelError("gated_add_layernorm wants contiguous float32 matrices of one shape")
+    T, H = h.shape
+    if H > GATED_ADD_NORM_MAX or weight.numel() != H or not weight.is_contiguous() \
+            or (bias is not None and (bias.numel() != H or bias.dtype != weight.dtype or not bias.is_contiguous())):
+        raise KernelError(f"gated_add_layernorm: rows of {H} columns (up to {GATED_ADD_NORM_MAX}) with weight and bias of one type")
+    out = torch.empty((T, H), dtype=out_dtype, device=h.device)
+    _call("elementwise", "fx_gated_add_layernorm", _stream(), dtype_code(out_dtype), _p(h), _p(y), _p(gate_logits), _p(weight),
+          _p(bias), dtype_code(weight.dtype), _p(out), T, H, float(eps))
+    return out
 
 
 def temp_unit_kv_write(qkv, q_out, positions, token_seq, block_table, k_pages, v_pages, n_heads: int, n_kv_heads: int,

@@ -193,19 +193,38 @@ class GatedPreNormBlock(Block):
             ops.fill_u32(out, 0)
             part.forward(x, ctx, *cache, out)
 
-    def _join(self, h, out, gate, x):
+    def _join(self, h, out, gate, x, ctx=None, then=None):
+        """The sublayer's rows through their gate into the stream.  `then`: the norm that reads the stream next; if it
+        offers `after_gated_add`, the add and that norm are one launch, and its rows are returned."""
         from .. import ops
         debug.region("residual gate")
         if gate is None:
             ops.residual_add(h, out)
-        else:
-            ops.gated_add(h, out, gate(x, epilogue=ops.EPI_STORE_F32))
+            return None
+        logits = gate(x, epilogue=ops.EPI_STORE_F32)
+        fused = getattr(then, "after_gated_add", None)
+        normed = fused(h, out, logits, ctx) if fused is not None else None
+        if normed is None:
+            ops.gated_add(h, out, logits)
+        return normed
 
-    def forward(self, h, ctx, cache):
+    chains_norms = True     # forward takes `normed` and `then` and returns what the next block may take as `normed`
+
+    @property
+    def first_norm(self):
+        return self.norm1
+
+    def forward(self, h, ctx, cache, normed=None, then=None):
+        """`normed`: norm1(h), if the block before has made it with the add that finished its rows.  `then`: (the
+        norm that the next block applies first, ...): this block's last gated add makes that norm's rows too, where
+        the norm offers it, and they are returned (else None)."""
         from .. import ops
         from .recurrent import sequence_starts
-        debug.region("norm")
-        x = self.norm1.forward(h, ctx)
+        after = then[0] if then is not None else None
+        x = normed
+        if x is None:
+            debug.region("norm")
+            x = self.norm1.forward(h, ctx)
         read = x
         if self.conv_taps:
             debug.region("input conv")
@@ -213,10 +232,11 @@ class GatedPreNormBlock(Block):
                                   ctx.n_seqs, activation=None, add_input=True, out_dtype=x.dtype)
         out = torch.empty_like(h)
         self._into(self.mixer, out, read, ctx, cache)
-        self._join(h, out, self.gate1, x)
+        x = self._join(h, out, self.gate1, x, ctx, self.norm2 if self.ffn is not None else after)
         if self.ffn is None:
-            return
-        debug.region("norm")
-        x = self.norm2.forward(h, ctx)
+            return x
+        if x is None:
+            debug.region("norm")
+            x = self.norm2.forward(h, ctx)
         self._into(self.ffn, out, x, ctx)
-        self._join(h, out, self.gate2, x)
+        return self._join(h, out, self.gate2, x, ctx, after)

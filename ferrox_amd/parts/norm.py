@@ -76,3 +76,10 @@ class LayerNorm(Norm):
 
     def forward(self, h, ctx, rows=None):
         return ops.layernorm(h, self.weight, self.bias, self.eps, ctx.act_dtype, rows=rows)
+
+    def after_gated_add(self, h, y, gate_logits, ctx):
+        """h += y * sigmoid(gate_logits), then this norm of the new rows, in one launch; None where the kernel does
+        not take the rows (the caller then does the two by themselves)."""
+        if self.size > ops.GATED_ADD_NORM_MAX:
+            return None
+        return ops.gated_add_layernorm(h, y, gate_logits, self.weight, self.bias, self.eps, ctx.act_dtype)

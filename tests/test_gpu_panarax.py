@@ -271,6 +271,10 @@ def test_layer_norm_gated_add_and_position_table(dtype):
     out = h.clone()
     ops.gated_add(out, y, g)
     assert torch.allclose(out.cpu().to(F64), h.cpu().to(F64) + y.cpu().to(F64) * plain.sigmoid(g.cpu().to(F64)), rtol=1e-6, atol=1e-6)
+    # the add and the norm behind it as one launch: the bits of the two launches
+    both = h.clone()
+    normed = ops.gated_add_layernorm(both, y, g, w, b, 1e-5, dtype)
+    assert torch.equal(both, out) and torch.equal(normed, ops.layernorm(out, w, b, 1e-5, dtype))
     table, pos = torch.randn(20, 70, generator=gen).to(dtype).cuda(), torch.randn(9, 70, generator=gen).to(dtype).cuda()
     ids = torch.tensor([3, 19, 0, 3], dtype=torch.int32, device="cuda")
     places = torch.tensor([0, 8, 2, 2], dtype=torch.int32, device="cuda")
